@@ -12,6 +12,12 @@ table per request and one buffer `[entries, pages, *page shape]` per declared te
 needs get `[slots, *shape]` buffers, zeroed when a slot is assigned.  A request holds one
 slot for its life; the slot is its row in every block table and state buffer.
 
+An entry that keeps several things (paged keys and values beside a convolution's last inputs, a
+matrix memory beside its normaliser) declares a dictionary name -> need, nested as deep as its
+parts are, and sees a dictionary of views of the same form.  An entry that reads another entry's
+cache may still keep state of its own: its view holds its own leaves, and the owner's leaves,
+not writable, wherever it has none of that name.
+
 The bookkeeping is host-side and works without a GPU (`device=None`), which is how the
 CPU tests drive it.  Reference: one pool, one table per slot, per-slot model state
 (crates/cuda-kernels/src/paged_kv.rs:34-102; infer/src/scheduler/cuda/core/construction.rs:119-203).
@@ -79,24 +85,44 @@ class PagedNeed:
 @dataclass(frozen=True)
 class StateNeed:
     shape: tuple
-    dtype: torch.dtype = torch.float32
+    dtype: torch.dtype | None = torch.float32   # None: the engine's activation type
 
-    def bytes_per_slot(self) -> int:
+    def bytes_per_slot(self, act_dtype: torch.dtype = torch.float32) -> int:
         n = 1
         for d in self.shape:
             n *= int(d)
-        return n * torch.empty((), dtype=self.dtype).element_size()
+        return n * torch.empty((), dtype=self.dtype or act_dtype).element_size()
+
+
+def need_leaves(need, path: tuple = ()) -> list:
+    """[(path, PagedNeed | StateNeed)] of one entry's need: itself at the empty path, or the leaves of a (nested)
+    dictionary of named needs."""
+    if need is None:
+        return []
+    if isinstance(need, dict):
+        out = []
+        for name, sub in need.items():
+            out += need_leaves(sub, path + (name,))
+        return out
+    if not isinstance(need, (PagedNeed, StateNeed)):
+        raise TypeError(f"a cache need is a PagedNeed, a StateNeed or a dictionary of them, not {type(need).__name__}")
+    return [(path, need)]
+
+
+def all_leaves(needs) -> list:
+    """Every leaf need of a model's entries, in entry order."""
+    return [leaf for need in needs for _, leaf in need_leaves(need)]
 
 
 def cache_bytes_per_token(needs, act_dtype: torch.dtype) -> int:
     """Bytes one token takes over every schedule entry that owns a paged cache.  For keys and values of every
     layer this is the reference's 2 * layers * kv_heads * head_dim * element size
     (infer/src/model/qwen3/forward.rs:777-783)."""
-    return sum(n.bytes_per_token(act_dtype) for n in needs if isinstance(n, PagedNeed))
+    return sum(n.bytes_per_token(act_dtype) for n in all_leaves(needs) if isinstance(n, PagedNeed))
 
 
-def state_bytes_per_slot(needs) -> int:
-    return sum(n.bytes_per_slot() for n in needs if isinstance(n, StateNeed))
+def state_bytes_per_slot(needs, act_dtype: torch.dtype = torch.float32) -> int:
+    return sum(n.bytes_per_slot(act_dtype) for n in all_leaves(needs) if isinstance(n, StateNeed))
 
 
 def pages_for_memory(free_bytes: int, total_bytes: int, mem_fraction_static: float, bytes_per_page: int,
@@ -149,6 +175,16 @@ class StateView:
     state: torch.Tensor | None     # [slots, *shape]
 
 
+def _merge_views(own, lent):
+    """A reader's view: its own leaves, and the owner's wherever it has none of that name."""
+    if isinstance(own, dict) and isinstance(lent, dict):
+        out = dict(own)
+        for name, sub in lent.items():
+            out[name] = _merge_views(own[name], sub) if name in own and own[name] is not None else sub
+        return out
+    return own if own is not None else lent
+
+
 class NoFreeSlot(RuntimeError):
     pass
 
@@ -176,8 +212,11 @@ class CacheManager:
         self.groups: list = []          # PageGroup
         self._group_needs: list = []    # PagedNeed of each group
         self._group_entries: list = []  # schedule entries of each group, in order
-        self._entry_place: dict = {}    # entry -> (group index, index within group)
-        for entry, need in enumerate(self.needs):
+        self._entry_place: dict = {}    # leaf key -> (group index, index within group)
+        # a leaf's key: the entry's index for a need that stands alone, (entry, *names) inside a dictionary
+        self._leaves = [(self._leaf_key(entry, path), leaf) for entry, whole in enumerate(self.needs)
+                        for path, leaf in need_leaves(whole)]
+        for entry, need in self._leaves:
             if isinstance(need, PagedNeed):
                 if need not in self._group_needs:
                     own = int(need.page_size or page_size)
@@ -217,10 +256,14 @@ class CacheManager:
                                         dtype=t.dtype or dtype, device=device)
                     for t in need.page_tensors()})
                 self.tables_dev.append(torch.zeros((max_slots, self._table_widths[g]), dtype=torch.int32, device=device))
-            for entry, need in enumerate(self.needs):
+            for entry, need in self._leaves:
                 if isinstance(need, StateNeed):
                     self.state_buffers[entry] = torch.zeros((max_slots, *need.shape),
-                                                            dtype=need.dtype, device=device)
+                                                            dtype=need.dtype or dtype, device=device)
+
+    @staticmethod
+    def _leaf_key(entry: int, path: tuple):
+        return (entry, *path) if path else entry
 
     # -- requests -------------------------------------------------------------------
     def admit(self, key) -> int:
@@ -349,17 +392,30 @@ class CacheManager:
             self._dirty[g].clear()
 
     def view(self, entry: int):
-        """The cache of a schedule entry: its own, or the one it was told to read."""
-        owner = self.readers.get(entry, entry)
-        need = self.needs[owner] if owner < len(self.needs) else None
+        """The cache of a schedule entry: its own, or the one it was told to read; for a dictionary of needs a
+        dictionary of views, in which a reader finds the owner's leaves (not writable) beside its own."""
+        own = self.needs[entry] if entry < len(self.needs) else None
+        tree = self._view_of(entry, own, (), True)
+        owner = self.readers.get(entry)
+        if owner is None:
+            return tree
+        lent = self._view_of(owner, self.needs[owner] if owner < len(self.needs) else None, (), False)
+        if tree is None:
+            return lent
+        return _merge_views(tree, lent)
+
+    def _view_of(self, entry: int, need, path: tuple, writes: bool):
+        if isinstance(need, dict):
+            return {name: self._view_of(entry, sub, path + (name,), writes) for name, sub in need.items()}
+        key = self._leaf_key(entry, path)
         if isinstance(need, PagedNeed):
-            g, idx = self._entry_place[owner]
+            g, idx = self._entry_place[key]
             has = self.device is not None
             pages = {t.name: (self.page_buffers[g][t.name][idx] if has else None) for t in need.page_tensors()}
             return PagedView(pages=pages, block_table=self.tables_dev[g] if has else None,
-                             page_size=self.groups[g].page_size, window=need.window, writes=owner == entry)
+                             page_size=self.groups[g].page_size, window=need.window, writes=writes)
         if isinstance(need, StateNeed):
-            return StateView(state=self.state_buffers.get(owner))
+            return StateView(state=self.state_buffers.get(key))
         return None
 
     def bytes_per_token(self) -> int:
@@ -386,4 +442,5 @@ class CacheManager:
 
 
 __all__ = ["CacheManager", "PagedNeed", "PageTensor", "PAGE", "StateNeed", "PagedView", "StateView", "OutOfPages",
-           "NoFreeSlot", "FREED", "cache_bytes_per_token", "state_bytes_per_slot", "pages_for_memory"]
+           "NoFreeSlot", "FREED", "cache_bytes_per_token", "state_bytes_per_slot", "pages_for_memory", "need_leaves",
+           "all_leaves"]

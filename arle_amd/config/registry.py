@@ -33,6 +33,8 @@ def known_architectures() -> list:
 
 def detect_architecture(raw: dict) -> Architecture:
     names = raw.get("architectures") if isinstance(raw, dict) else None
+    if names is None and isinstance(raw, dict) and isinstance(raw.get("architecture"), str):
+        names = [raw["architecture"]]     # a design that names itself with one string
     if names is None:
         raise ConfigError("config.json has no `architectures` field")
     if not isinstance(names, list) or not all(isinstance(n, str) for n in names):

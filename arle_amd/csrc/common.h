@@ -89,6 +89,19 @@ __device__ __forceinline__ float block_max(float v, float* lds /* [kWaves] */) {
   return total;
 }
 
+// Element access by a run-time type code (kF32 / kBF16 below), for operands whose type follows the checkpoint
+// or the engine's mode and whose kernels are bound by memory: the branch is the same in every lane.
+__device__ __forceinline__ float load_as_float(const void* p, int code, int64_t i) {
+  return code == 0 ? static_cast<const float*>(p)[i] : to_float(static_cast<const bf16*>(p)[i]);
+}
+__device__ __forceinline__ void store_from_float(void* p, int code, int64_t i, float v) {
+  if (code == 0) {
+    static_cast<float*>(p)[i] = v;
+  } else {
+    static_cast<bf16*>(p)[i] = from_float<bf16>(v);
+  }
+}
+
 inline int launch_status() { return static_cast<int>(hipGetLastError()); }
 
 // Element type codes shared with the Python side.

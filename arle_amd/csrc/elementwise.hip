@@ -1,6 +1,6 @@
 // Embedding gather and the SiLU-gated product.
 //
-// embed_gather: out[t, :] = float(table[ids[t], :])      (residual stream is 32-bit)
+// embed_gather: out[t, :] = float(table[ids[t], :]) * scale   (residual stream is 32-bit; scale 1 for most models)
 //   reference counterpart: crates/cuda-kernels/csrc/misc/elementwise_basic.cu:186-211
 // silu_mul:     out[t, j] = silu(gate[t, j]) * up[t, j], silu(z) = z / (1 + exp(-z))
 //   reference counterpart: crates/cuda-kernels/csrc/misc/elementwise_basic.cu:18-24,34-95
@@ -10,11 +10,11 @@ namespace arle {
 
 template <typename TT>
 __global__ void embed_gather_kernel(const TT* __restrict__ table, const int* __restrict__ ids,
-                                    float* __restrict__ out, int hidden) {
+                                    float* __restrict__ out, int hidden, float scale) {
   const int t = blockIdx.x;
   const TT* src = table + static_cast<int64_t>(ids[t]) * hidden;
   float* dst = out + static_cast<int64_t>(t) * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]) * scale;
 }
 
 // block == 0: gate and up are two [T, width] views.  block > 0: one buffer whose columns alternate
@@ -104,13 +104,13 @@ __global__ __launch_bounds__(256) void sum_partials_x4_kernel(const float* __res
 using namespace arle;
 
 extern "C" int arle_embed_gather(const void* table, int table_dtype, const int* ids, float* out,
-                                 int tokens, int hidden, void* stream) {
+                                 int tokens, int hidden, float scale, void* stream) {
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (table_dtype == kF32) {
-    embed_gather_kernel<float><<<tokens, 256, 0, s>>>(static_cast<const float*>(table), ids, out, hidden);
+    embed_gather_kernel<float><<<tokens, 256, 0, s>>>(static_cast<const float*>(table), ids, out, hidden, scale);
   } else {
-    embed_gather_kernel<bf16><<<tokens, 256, 0, s>>>(static_cast<const bf16*>(table), ids, out, hidden);
+    embed_gather_kernel<bf16><<<tokens, 256, 0, s>>>(static_cast<const bf16*>(table), ids, out, hidden, scale);
   }
   return launch_status();
 }

@@ -15,8 +15,8 @@ import os
 import torch
 
 from .. import models  # noqa: F401  (registers the architectures)
-from ..cache.manager import (CacheManager, OutOfPages, PagedNeed, cache_bytes_per_token, pages_for_memory, slots_for_tokens,
-                             state_bytes_per_slot)
+from ..cache.manager import (CacheManager, OutOfPages, PagedNeed, all_leaves, cache_bytes_per_token, pages_for_memory,
+                             slots_for_tokens, state_bytes_per_slot)
 from ..config.registry import detect_architecture, load_model_config
 from ..models.decoder import DEBUG_DUMP_ENV, build_model, expected_checkpoint_tensors
 from ..parts.base import Runtime
@@ -113,9 +113,9 @@ class Engine:
             longest = min(max_request_tokens or spec.max_positions, spec.max_positions)
             free, total = torch.cuda.mem_get_info(self.device)
             num_pages = pages_for_memory(free, total, mem_fraction_static, self.kv_bytes_per_token * page_size,
-                                         reserved_bytes=max_slots * state_bytes_per_slot(needs),
+                                         reserved_bytes=max_slots * state_bytes_per_slot(needs, self.dtype),
                                          most_pages=max_slots * -(-longest // page_size))
-            if num_pages < 1 and any(isinstance(n, PagedNeed) for n in needs):
+            if num_pages < 1 and any(isinstance(n, PagedNeed) for n in all_leaves(needs)):
                 raise EngineError(f"no memory for the cache: {free / 2**30:.1f} GiB are free, the headroom of "
                                   f"{(1 - mem_fraction_static) * 100:.0f} % of {total / 2**30:.1f} GiB leaves less than "
                                   f"one page of {self.kv_bytes_per_token * page_size} bytes")

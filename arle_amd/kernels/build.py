@@ -34,6 +34,11 @@ SOURCES = {
     "attention_mfma": "attention_mfma.hip",
     "sampling": "sampling.hip",
     "ceilings": "ceilings.hip",
+    "layernorm": "layernorm.hip",
+    "short_conv": "short_conv.hip",
+    "polynorm": "polynorm.hip",
+    "mlstm": "mlstm.hip",
+    "attention_softcap": "attention_softcap.hip",
     "host": "host/runtime.cpp",
 }
 HEADERS = ("common.h", "attention_static.h", "attention_args.h", "attention_stream.h", "attention_portions.h",

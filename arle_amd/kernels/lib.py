@@ -19,7 +19,7 @@ _f = ctypes.c_float
 
 # function name -> (library, argument types); every function returns a hipError_t as int
 SIGNATURES = {
-    "arle_embed_gather": ("elementwise", [_p, _i, _p, _p, _i, _i, _p]),
+    "arle_embed_gather": ("elementwise", [_p, _i, _p, _p, _i, _i, _f, _p]),
     "arle_silu_mul": ("elementwise", [_p, _p, _ll, _p, _i, _i, _i, _i, _p]),
     "arle_rmsnorm": ("norm", [_p, _i, _ll, _p, _i, _p, _i, _p, _i, _i, _f, _p]),
     "arle_add_rmsnorm": ("norm", [_p, _p, _i, _ll, _i, _p, _i, _p, _i, _p, _i, _i, _f, _p]),
@@ -57,6 +57,18 @@ SIGNATURES = {
     "arle_token_logprobs": ("sampling", [_p, _i, _i, _p, _p, _p]),
     "arle_attn_decode_static": ("attention_mfma", [_p, _ll, _p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i,
                                                    _i, _f, _i, _i, _p]),
+    "arle_add_layernorm": ("layernorm", [_p, _p, _i, _ll, _i, _p, _i, _p, _i, _ll, _i, _p, _i, _p, _p, _i, _p, _p, _i, _p, _i,
+                                         _i, _f, _p]),
+    "arle_causal_conv": ("short_conv", [_p, _ll, _i, _p, _i, _p, _i, _p, _i, _p, _p, _ll, _i, _i, _i, _i, _i, _p]),
+    "arle_conv_state_update": ("short_conv", [_p, _ll, _i, _p, _i, _p, _i, _p, _p, _i, _i, _i, _p]),
+    "arle_polynorm": ("polynorm", [_p, _ll, _i, _p, _i, _p, _i, _p, _i, _i, _i, _f, _p]),
+    "arle_mlstm_scan": ("mlstm", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _ll, _p, _p, _i, _f, _p, _p, _p, _p, _p, _i, _p, _p,
+                                  _i, _i, _i, _p]),
+    "arle_mlstm_output": ("mlstm", [_p, _p, _ll, _i, _p, _i, _p, _i, _i, _i, _i, _f, _p]),
+    "arle_qkv_norm_store": ("attention_softcap", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _f, _f, _i, _p, _p, _p, _i,
+                                                  _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "arle_attn_softcap_simt": ("attention_softcap", [_p, _ll, _p, _ll, _p, _p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i,
+                                                     _f, _f, _p, _p, _i, _i, _p]),
     "arle_ceiling_read": ("ceilings", [_p, _ll, _i, _p, _p, _p]),
     "arle_ceiling_mfma": ("ceilings", [_i, _i, _i, _i, _p, _p]),
 }

@@ -74,8 +74,8 @@ def _ptr(t) -> int:
 # ------------------------------------------------------------------ embedding
 
 
-def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None):
-    """out[t, :] = float32(table[ids[t], :]).  ids must already be checked to lie in range."""
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None, scale: float = 1.0):
+    """out[t, :] = float32(table[ids[t], :]) * scale.  ids must already be checked to lie in range."""
     _gpu(table, ids, out)
     _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [V, H]")
     _i32(ids, "ids")
@@ -85,7 +85,7 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | Non
     _need(out.dtype == torch.float32 and out.shape == (tokens, hidden) and out.is_contiguous(),
           "embed_gather output must be contiguous float32 [T, H]")
     lib.call("arle_embed_gather", table.data_ptr(), _code(table), ids.data_ptr(), out.data_ptr(),
-             tokens, hidden, _stream())
+             tokens, hidden, float(scale), _stream())
     return out
 
 
@@ -1383,3 +1383,258 @@ if os.environ.get(PRODUCT_TABLE_ENV, "") != "none":
     load_shipped_product_tables()
     if os.environ.get(PRODUCT_TABLE_ENV):
         load_product_table(os.environ[PRODUCT_TABLE_ENV])
+
+
+# ------------------------------------------------- layer norm with the adds of a parallel block
+
+
+def _term_args(term, bias, shape):
+    """(pointer, stack depth, stack stride, type code, bias pointer, bias type code) of one addend of add_layernorm."""
+    if term is None:
+        _need(bias is None, "a bias without its term")
+        return (0, 0, 0, 0, 0, 0)
+    _need(term.dim() in (2, 3) and tuple(term.shape[-2:]) == tuple(shape) and term.is_contiguous() and term.dtype in _CODES,
+          "an addend must match the residual ([T, H] or a float32 stack [S, T, H])")
+    _need(term.dim() == 2 or (term.dtype == torch.float32 and term.shape[0] >= 1), "a stack of partial sums is float32")
+    if bias is not None:
+        _need(bias.shape == (shape[1],) and bias.is_contiguous() and bias.dtype in _CODES, "an addend's bias must be [H]")
+    return (term.data_ptr(), term.shape[0] if term.dim() == 3 else 1, shape[0] * shape[1], _code(term),
+            _ptr(bias), _code(bias) if bias is not None else 0)
+
+
+LAYERNORM_MAX_WIDTH = 16384
+
+
+def add_layernorm(residual: torch.Tensor, terms, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                  weight_b: torch.Tensor | None = None, rows: torch.Tensor | None = None):
+    """residual += sum of `terms` (float32, in place unless `rows` is given); then the layer norm without bias of
+    every row (or of the rows named by `rows`), once with `weight` and, if given, once more with `weight_b`.
+
+    terms: up to two (tensor, bias or None); a tensor is [T, H] or a float32 stack [S, T, H] added in order.
+    Returns out, or (out, out_b)."""
+    terms = list(terms or [])
+    _need(len(terms) <= 2, "add_layernorm adds at most two terms")
+    _gpu(residual, weight, weight_b, rows, *[t for pair in terms for t in pair])
+    _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
+          "residual must be contiguous float32 [T, H]")
+    width = residual.shape[1]
+    _need(0 < width <= LAYERNORM_MAX_WIDTH, f"layer norm takes widths up to {LAYERNORM_MAX_WIDTH}")
+    _need(weight.shape == (width,) and weight.is_contiguous(), "norm weight must be [width]")
+    if weight_b is not None:
+        _need(weight_b.shape == (width,) and weight_b.is_contiguous() and weight_b.dtype == weight.dtype,
+              "the second norm weight must be [width] of the first one's type")
+    n_rows = residual.shape[0]
+    if rows is not None:
+        _i32(rows, "rows")
+        n_rows = rows.numel()
+    out = torch.empty((n_rows, width), dtype=out_dtype, device=residual.device)
+    out_b = torch.empty_like(out) if weight_b is not None else None
+    args = []
+    for i in range(2):
+        args += _term_args(*(terms[i] if i < len(terms) else (None, None)), residual.shape)
+    lib.call("arle_add_layernorm", residual.data_ptr(), *args, weight.data_ptr(), _ptr(weight_b), _code(weight),
+             out.data_ptr(), _ptr(out_b), _code(out), _ptr(rows), n_rows, width, float(eps), _stream())
+    return out if weight_b is None else (out, out_b)
+
+
+# ------------------------------------------------------------- short causal convolution with state
+
+CONV_MAX_TAPS = 16
+
+
+def causal_conv(u: torch.Tensor, weight, state, slot_of_token: torch.Tensor, *, bias=None, add_input: bool = False,
+                out_dtype: torch.dtype | None = None):
+    """y_t = (u_t if add_input) + sum_j weight[:, j] * u_(t - taps + 1 + j) per channel, over the rows of each request
+    (consecutive in u) and, further back, over its state [slots, taps-1, C]; u counts with `bias` added.  weight
+    None: y = u + bias.  The state is not changed: `conv_state_update` does that once the step's rows are done."""
+    _gpu(u, weight, state, slot_of_token, bias)
+    _rows(u, "u")
+    tokens, channels = u.shape
+    _i32(slot_of_token, "slot_of_token", tokens)
+    taps = 1
+    if weight is not None:
+        _need(weight.dim() == 2 and weight.shape[0] == channels and weight.is_contiguous() and weight.dtype in _CODES,
+              "a convolution weight must be contiguous [channels, taps]")
+        taps = weight.shape[1]
+        _need(1 <= taps <= CONV_MAX_TAPS, f"the short convolution takes 1..{CONV_MAX_TAPS} taps")
+        if taps > 1:
+            _need(state is not None and state.dim() == 3 and tuple(state.shape[1:]) == (taps - 1, channels)
+                  and state.is_contiguous() and state.dtype in _CODES, "conv state must be [slots, taps-1, channels]")
+    if bias is not None:
+        _need(bias.shape == (channels,) and bias.is_contiguous() and bias.dtype in _CODES, "conv bias must be [channels]")
+    out = torch.empty((tokens, channels), dtype=out_dtype or u.dtype, device=u.device)
+    has_state = weight is not None and taps > 1
+    lib.call("arle_causal_conv", u.data_ptr(), u.stride(0), _code(u), _ptr(bias), _code(bias) if bias is not None else 0,
+             _ptr(weight), _code(weight) if weight is not None else 0, state.data_ptr() if has_state else 0,
+             _code(state) if has_state else 0, slot_of_token.data_ptr(), out.data_ptr(), out.stride(0), _code(out),
+             tokens, channels, taps, 1 if add_input else 0, _stream())
+    return out
+
+
+def conv_state_update(u: torch.Tensor, state: torch.Tensor, seg_row0: torch.Tensor, seg_slot: torch.Tensor, *, bias=None):
+    """state[slot] <- the last taps-1 rows of (state[slot], the request's rows of u (+ bias)), for every segment."""
+    _gpu(u, state, seg_row0, seg_slot, bias)
+    _rows(u, "u")
+    channels = u.shape[1]
+    _need(state.dim() == 3 and state.shape[2] == channels and state.is_contiguous() and state.dtype in _CODES
+          and state.shape[1] < CONV_MAX_TAPS, "conv state must be [slots, taps-1, channels]")
+    segments = seg_slot.numel()
+    _i32(seg_slot, "seg_slot")
+    _i32(seg_row0, "seg_row0", segments + 1)
+    lib.call("arle_conv_state_update", u.data_ptr(), u.stride(0), _code(u), _ptr(bias),
+             _code(bias) if bias is not None else 0, state.data_ptr(), _code(state), seg_row0.data_ptr(),
+             seg_slot.data_ptr(), segments, channels, state.shape[1] + 1, _stream())
+
+
+# ------------------------------------------------------------------------ PolyNorm activation
+
+
+def polynorm(u: torch.Tensor, coef: torch.Tensor, eps: float, *, bias=None, out_dtype: torch.dtype | None = None):
+    """a N(z) + b N(z^2) + c N(z^3) + e over rows of z = u + bias; N divides a row by its root mean square;
+    coef = (a, b, c, e) on the GPU."""
+    _gpu(u, coef, bias)
+    _rows(u, "u")
+    tokens, width = u.shape
+    _need(coef.shape == (4,) and coef.is_contiguous() and coef.dtype in _CODES, "PolyNorm takes four coefficients")
+    _need(0 < width <= 24576, "PolyNorm takes rows of up to 24,576 values")
+    if bias is not None:
+        _need(bias.shape == (width,) and bias.is_contiguous() and bias.dtype in _CODES, "the bias must be [width]")
+    out = torch.empty((tokens, width), dtype=out_dtype or u.dtype, device=u.device)
+    lib.call("arle_polynorm", u.data_ptr(), u.stride(0), _code(u), _ptr(bias), _code(bias) if bias is not None else 0,
+             coef.data_ptr(), _code(coef), out.data_ptr(), _code(out), tokens, width, float(eps), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------ mLSTM matrix memory
+
+MLSTM_MAX_KEY_DIM = 256
+
+
+def mlstm_scan(q, k, v, gates, bias_i, bias_f, cap: float, s_state, n_state, m_state, seg_row0, seg_slot, *,
+               heads: int, key_dim: int, value_dim: int):
+    """The matrix-memory recurrence over the rows of every segment, from and into the requests' states; returns
+    float32 [T, heads * value_dim]: S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6) with q scaled by
+    key_dim^(-1/2).  gates float32 [T, 2 * heads]: pre-activations of the input gates, then of the forget gates."""
+    _gpu(q, k, v, gates, bias_i, bias_f, s_state, n_state, m_state, seg_row0, seg_slot)
+    H, D, Dv = heads, key_dim, value_dim
+    tokens = q.shape[0]
+    for name, t, width in (("q", q, H * D), ("k", k, H * D), ("v", v, H * Dv)):
+        _rows(t, name)
+        _need(t.shape == (tokens, width) and t.dtype == q.dtype, f"{name} must be [T, {width}] of one type")
+    _need(0 < D <= MLSTM_MAX_KEY_DIM, f"the mLSTM kernels take key sizes up to {MLSTM_MAX_KEY_DIM}")
+    _rows(gates, "gates")
+    _need(gates.dtype == torch.float32 and gates.shape == (tokens, 2 * H), "gates must be float32 [T, 2 * heads]")
+    _need(bias_i.shape == (H,) and bias_f.shape == (H,) and bias_i.dtype == bias_f.dtype and bias_i.is_contiguous()
+          and bias_f.is_contiguous(), "gate biases must be [heads] of one type")
+    slots = s_state.shape[0]
+    _need(s_state.shape == (slots, H, D, Dv) and n_state.shape == (slots, H, D) and m_state.shape == (slots, H)
+          and all(t.dtype == torch.float32 and t.is_contiguous() for t in (s_state, n_state, m_state)),
+          "mLSTM states are float32 [slots, H, D, Dv], [slots, H, D] and [slots, H]")
+    segments = seg_slot.numel()
+    _i32(seg_slot, "seg_slot")
+    _i32(seg_row0, "seg_row0", segments + 1)
+    coefs = torch.empty((tokens, H, 3), dtype=torch.float32, device=q.device)
+    o = torch.empty((tokens, H * Dv), dtype=torch.float32, device=q.device)
+    lib.call("arle_mlstm_scan", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), _code(q),
+             gates.data_ptr(), gates.stride(0), bias_i.data_ptr(), bias_f.data_ptr(), _code(bias_i), float(cap),
+             s_state.data_ptr(), n_state.data_ptr(), m_state.data_ptr(), seg_row0.data_ptr(), seg_slot.data_ptr(),
+             segments, coefs.data_ptr(), o.data_ptr(), H, D, Dv, _stream())
+    return o
+
+
+def mlstm_output(o, gate, weight, eps: float, out_dtype, *, heads: int, value_dim: int):
+    """Each head's o divided by its root mean square, times `weight` [heads * value_dim], times sigmoid(gate)."""
+    _gpu(o, gate, weight)
+    tokens = o.shape[0]
+    width = heads * value_dim
+    _need(o.dtype == torch.float32 and o.shape == (tokens, width) and o.is_contiguous(), "o must be float32 [T, H * Dv]")
+    _rows(gate, "gate")
+    _need(gate.shape == (tokens, width) and gate.dtype in _CODES, "gate must be [T, H * Dv]")
+    _need(weight.shape == (width,) and weight.is_contiguous() and weight.dtype in _CODES, "the norm weight must be [H * Dv]")
+    out = torch.empty((tokens, width), dtype=out_dtype, device=o.device)
+    lib.call("arle_mlstm_output", o.data_ptr(), gate.data_ptr(), gate.stride(0), _code(gate), weight.data_ptr(),
+             _code(weight), out.data_ptr(), _code(out), tokens, heads, value_dim, float(eps), _stream())
+    return out
+
+
+# --------------------------------------------------- soft-capped attention with a distance penalty
+
+
+def _check_kv_pages(k_pages, v_pages, nkv, page_size, Dk, Dv, dtype):
+    _need(k_pages.dim() == 4 and tuple(k_pages.shape[1:]) == (nkv, page_size, Dk) and k_pages.is_contiguous()
+          and k_pages.dtype == dtype, "k_pages must be contiguous [pages, nkv, page_size, Dk]")
+    _need(v_pages.dim() == 4 and tuple(v_pages.shape[1:]) == (nkv, Dv, page_size) and v_pages.is_contiguous()
+          and v_pages.dtype == dtype and v_pages.shape[0] == k_pages.shape[0],
+          "v_pages must be contiguous [pages, nkv, Dv, page_size]")
+
+
+def qkv_norm_store(q, k, v, *, num_q_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, eps: float,
+                   q_weight=None, k_weight=None, temp_coef: float = 0.0, temp_every: int = 1, positions=None,
+                   slot_of_token=None, block_table=None, k_pages=None, v_pages=None, page_size: int = 0):
+    """Per-head RMS norm of q (in place, then times 1 + temp_coef ln(floor((p + 1) / temp_every) + 1)) and of k;
+    k and v go to the pages.  num_kv_heads 0 (k, v None): only q, for a layer that reads another layer's pages."""
+    _gpu(q, k, v, q_weight, k_weight, positions, slot_of_token, block_table, k_pages, v_pages)
+    tokens = q.shape[0]
+    _rows(q, "q")
+    _need(q.shape == (tokens, num_q_heads * key_dim) and q.dtype in _CODES, "q must be [T, heads * Dk]")
+    _need(0 < key_dim <= MAX_HEAD_DIM and 0 < value_dim, "head sizes out of range")
+    _i32(positions, "positions", tokens)
+    w_code = 0
+    for w in (q_weight, k_weight):
+        if w is not None:
+            _need(w.shape == (key_dim,) and w.is_contiguous() and w.dtype in _CODES, "a q/k norm weight must be [Dk]")
+            w_code = _code(w)
+    if q_weight is not None and k_weight is not None:
+        _need(q_weight.dtype == k_weight.dtype, "q and k norm weights must be of one type")
+    table_stride = 0
+    if num_kv_heads:
+        _rows(k, "k")
+        _rows(v, "v")
+        _need(k.shape == (tokens, num_kv_heads * key_dim) and v.shape == (tokens, num_kv_heads * value_dim)
+              and k.dtype == q.dtype and v.dtype == q.dtype, "k, v must be [T, kv heads * Dk], [T, kv heads * Dv]")
+        _check_kv_pages(k_pages, v_pages, num_kv_heads, page_size, key_dim, value_dim, q.dtype)
+        _i32(slot_of_token, "slot_of_token", tokens)
+        _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+              "block_table must be contiguous int32 [slots, pages]")
+        table_stride = block_table.shape[1]
+    _need(temp_coef == 0.0 or temp_every >= 1, "the query temperature's period must be positive")
+    kk, vv = (k, v) if num_kv_heads else (q, q)
+    lib.call("arle_qkv_norm_store", q.data_ptr(), q.stride(0), kk.data_ptr(), kk.stride(0), vv.data_ptr(), vv.stride(0),
+             _code(q), _ptr(q_weight), _ptr(k_weight), w_code, float(eps), float(temp_coef), int(temp_every),
+             positions.data_ptr(), _ptr(slot_of_token) if num_kv_heads else 0, _ptr(block_table) if num_kv_heads else 0,
+             table_stride, _ptr(k_pages) if num_kv_heads else 0, _ptr(v_pages) if num_kv_heads else 0, tokens,
+             num_q_heads, num_kv_heads, key_dim, value_dim, int(page_size), _stream())
+
+
+def attn_softcap_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_token, *, num_q_heads: int,
+                      num_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
+                      softcap: float = 0.0, r1=None, r2=None, window: int = 0):
+    """Causal attention of every row over its request's pages: scores scale (q . k), soft-capped (softcap > 0), less
+    r1_h ln(1 + r2_h distance) (r1, r2 [heads] given), over the last `window` keys (0: all)."""
+    _gpu(q, out, k_pages, v_pages, block_table, positions, slot_of_token, r1, r2)
+    tokens = q.shape[0]
+    _rows(q, "q")
+    _rows(out, "out")
+    _need(q.shape == (tokens, num_q_heads * key_dim) and out.shape == (tokens, num_q_heads * value_dim)
+          and out.dtype == q.dtype, "q [T, nq*Dk] and out [T, nq*Dv] must be of one type")
+    _need(num_kv_heads > 0 and num_q_heads % num_kv_heads == 0, "number of q heads must be a multiple of the kv heads")
+    _need(max(key_dim, value_dim) <= MAX_HEAD_DIM and num_q_heads <= _GRID_Y_MAX, "head sizes or counts out of range")
+    _check_kv_pages(k_pages, v_pages, num_kv_heads, page_size, key_dim, value_dim, q.dtype)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [slots, pages]")
+    _i32(positions, "positions", tokens)
+    _i32(slot_of_token, "slot_of_token", tokens)
+    _need((r1 is None) == (r2 is None), "give both distance constants or neither")
+    if r1 is not None:
+        _need(r1.shape == (num_q_heads,) and r2.shape == (num_q_heads,) and r1.dtype == r2.dtype and r1.dtype in _CODES
+              and r1.is_contiguous() and r2.is_contiguous(), "r1, r2 must be [heads] of one type")
+    lib.call("arle_attn_softcap_simt", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(),
+             v_pages.data_ptr(), _code(q), block_table.data_ptr(), block_table.shape[1], positions.data_ptr(),
+             slot_of_token.data_ptr(), tokens, num_q_heads, num_kv_heads, key_dim, value_dim, page_size, float(scale),
+             float(softcap), _ptr(r1), _ptr(r2), _code(r1) if r1 is not None else 0, int(window), _stream())
+    return out
+
+
+def attn_softcap_mfma_supported(dtype, key_dim: int, value_dim: int, page_size: int, group: int) -> bool:
+    """Whether the matrix-core kernel of the soft-capped attention takes this shape."""
+    return False

@@ -12,7 +12,8 @@ import sys
 
 from ..kernels import ops
 from ..parts import base  # noqa: F401  (registries)
-from ..parts import attention, block, embedding, feed_forward, norm, position  # noqa: F401  registers the stock parts
+from ..parts import (attention, block, embedding, feed_forward, mlstm, norm, position,  # noqa: F401  registers the stock parts
+                     short_conv, softcap_attention)
 from ..parts.base import Runtime, build_part, expected_tensors, lookup
 from ..parts.spec import ModelSpec
 
@@ -47,11 +48,13 @@ def declared_cache_needs(spec: ModelSpec) -> list:
     weights, no GPU): what a shape summary and a memory plan are made from."""
     needs = []
     for entry in spec.schedule:
-        if entry.cache_from is not None:
+        mixer = spec.layers[entry.layer].mixer
+        if mixer is None:
             needs.append(None)
+        elif entry.cache_from is not None:
+            needs.append(lookup("mixer", mixer.kind).declare_reader_cache(mixer.params))
         else:
-            mixer = spec.layers[entry.layer].mixer
-            needs.append(None if mixer is None else lookup("mixer", mixer.kind).declare_cache(mixer.params))
+            needs.append(lookup("mixer", mixer.kind).declare_cache(mixer.params))
     return needs
 
 
@@ -72,8 +75,11 @@ def debug_dump(residual, delta, label: str) -> None:
     reference prints with INFER_DEBUG_DUMP (infer/src/model/common.rs:85-124).  Synchronises; steps are then not
     captured."""
     row = residual[-1].float()
-    if delta is not None:
-        row = row + (delta.float().sum(0) if delta.dim() == 3 else delta.float())[-1]
+    terms = delta if isinstance(delta, list) else ([] if delta is None else [(delta, None)])
+    for term, bias in terms:
+        row = row + (term.float().sum(0) if term.dim() == 3 else term.float())[-1]
+        if bias is not None:
+            row = row + bias.float()
     row = row.cpu()
     fmt = lambda vals: "[" + ", ".join(f"{v:+.5f}" for v in vals.tolist()) + "]"
     print(f"[debug-dump] {label}: head={fmt(row[:8])} tail={fmt(row[-4:])} min={float(row.min()):.4f} "
@@ -130,11 +136,12 @@ class DecoderModel:
         """(need of every schedule entry that owns a cache, {reader entry -> owner entry})."""
         needs, readers = [], {}
         for i, entry in enumerate(self.schedule):
+            mixer = self.blocks[entry.layer].mixer
             if entry.cache_from is not None:
-                needs.append(None)
+                own = getattr(mixer, "reader_cache_need", None)     # state it keeps beside the cache it borrows
+                needs.append(own() if own is not None else None)
                 readers[i] = entry.cache_from
             else:
-                mixer = self.blocks[entry.layer].mixer
                 needs.append(mixer.cache_need() if mixer is not None else None)
         return needs, readers
 

@@ -12,12 +12,14 @@ Interfaces (T = tokens of the packed step, H = hidden size, A = activation dtype
                 A delta is A[T,H], or a float32 stack [S,T,H] of partial sums to be added in the order
                 of S (what a matrix product with K split over workgroups leaves behind).
 * position      `fused_rotary() -> (cos, sin, rotary_dim) | None`;  `apply(q, k, positions)` in place.
-* mixer         `cache_need() -> PagedNeed | StateNeed | None` (and, so that a model's cache can be sized
-                from its description alone, the class method `declare_cache(params)` with the same answer);
-                `forward(x A[T,H], batch: StepBatch, cache_view) -> delta`.
+* mixer         `cache_need() -> PagedNeed | StateNeed | {name: need, ...} | None` (and, so that a model's cache can
+                be sized from its description alone, the class method `declare_cache(params)` with the same answer;
+                `reader_cache_need()` / `declare_reader_cache(params)`: what it keeps in an entry that reads another
+                entry's cache); `forward(x A[T,H], batch: StepBatch, cache_view) -> delta`.
 * feed_forward  `forward(x A[T,H]) -> delta`.
 * block         `forward(residual f32[T,H], delta | None, batch, cache_view) -> (residual, delta)`;
-                the returned delta is what the next block (or the final norm) still has to add.
+                the returned delta is what the next block (or the final norm) still has to add: a tensor, a stack,
+                or a `Pending` list of (tensor or stack, bias or None) for norms that add several terms in one pass.
 * embedding     `forward(token_ids i32[T]) -> f32[T,H]`.
 * head          `forward(x A[R,H]) -> f32[R,V]`.
 """
@@ -73,6 +75,10 @@ class Runtime:
         return self.act_dtype == torch.float32
 
 
+class Pending(list):
+    """What a block leaves for the next norm to add into the residual: [(tensor or float32 stack, bias or None), ...]."""
+
+
 class Part:
     role = ""
     kind = ""
@@ -96,6 +102,15 @@ class Part:
         """What a mixer of these sizes keeps between steps (PagedNeed | StateNeed | None), known without building
         it.  A mixer that only answers `cache_need()` on a built instance is sized from the built model."""
         return None
+
+    @classmethod
+    def declare_reader_cache(cls, params: dict):
+        """What a mixer of these sizes still keeps for itself in an entry that reads another entry's cache (state of
+        its own beside the pages it borrows); None: nothing."""
+        return None
+
+    def reader_cache_need(self):
+        return self.declare_reader_cache(self.params)
 
     def __init__(self, params: dict, tensors: dict, rt: Runtime, children: dict | None = None):
         self.params = params
@@ -161,5 +176,5 @@ def build_part(role: str, spec: PartSpec, fetch, rt: Runtime):
     return cls(spec.params, tensors, rt, kids)
 
 
-__all__ = ["register", "lookup", "Runtime", "Part", "expected_tensors", "build_part", "WeightDecl",
+__all__ = ["register", "lookup", "Runtime", "Part", "Pending", "expected_tensors", "build_part", "WeightDecl",
            "PartSpec", "Rows", "UnknownPart", "ROLES"]

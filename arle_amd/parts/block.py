@@ -28,3 +28,34 @@ class PreNormBlock:
         m = self.mixer.forward(a, batch, cache_view)
         b = self.norm_ffn.add_norm(residual, m)
         return residual, self.feed_forward.forward(b)
+
+
+@register("block", "parallel")
+class ParallelBlock:
+    """h += mixer(norm_a(h)) + ffn(norm_b(h)): both read the same residual.  norm roles: "mixer_in", "ffn_in" (the
+    second only with a feed-forward).  The two outputs go on, unadded, to the next block's norms (or the final one),
+    which add them in the pass that computes their statistics; the two norms of this block come out of one pass too.
+    A mixer or feed-forward may hand back (delta, bias): the bias of its last projection, added with the delta."""
+
+    norm_roles = ("mixer_in", "ffn_in")
+
+    def __init__(self, mixer, feed_forward, norms: dict):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norms = norms
+        self.norm_mixer = norms["mixer_in"]
+        self.norm_ffn = norms.get("ffn_in") if feed_forward is not None else None
+
+    def forward(self, residual, delta, batch, cache_view):
+        from .base import Pending
+
+        if self.norm_ffn is not None:
+            a, b = self.norm_mixer.add_norm(residual, delta, also=self.norm_ffn)
+        else:
+            a = self.norm_mixer.add_norm(residual, delta)
+        left = Pending()
+        for out in (self.mixer.forward(a, batch, cache_view),
+                    self.feed_forward.forward(b) if self.norm_ffn is not None else None):
+            if out is not None:
+                left.append(out if isinstance(out, tuple) else (out, None))
+        return residual, left

@@ -14,7 +14,7 @@ from .linear import Linear
 
 @register("embedding", "token_table")
 class TokenEmbedding(Part):
-    """params: vocab_size, hidden_size."""
+    """params: vocab_size, hidden_size, scale (a factor on every row, in 32 bits; default 1)."""
 
     graph_safe = True  # launches depend on shapes only, never on the values of a step
 
@@ -25,9 +25,10 @@ class TokenEmbedding(Part):
     def __init__(self, params, tensors, rt, children=None):
         super().__init__(params, tensors, rt, children)
         self.table = tensors["table"]
+        self.scale = float(params.get("scale", 1.0))
 
     def forward(self, token_ids):
-        return ops.embed_gather(self.table, token_ids)
+        return ops.embed_gather(self.table, token_ids, scale=self.scale)
 
 
 @register("head", "linear")

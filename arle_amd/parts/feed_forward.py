@@ -1,4 +1,5 @@
-"""Dense SwiGLU feed-forward: down(silu(gate(x)) * up(x)), no biases.
+"""Dense feed-forwards.  SwiGLU: down(silu(gate(x)) * up(x)), no biases; PolyNorm (below): one projection up
+with a bias, a polynomial of row-normalised powers, one projection down with a bias.
 
 infer/src/model/qwen3/prefill.rs:291-337.  gate and up are kept as one [2I, H] matrix
 (gate rows first, as the reference's optional fusion does, weights.rs:111-121) so a step
@@ -56,3 +57,36 @@ class SwiGLU(Part):
             gu = self.gate_up(x)
             act = ops.silu_mul(gu[:, : self.inter], gu[:, self.inter:])
         return self.down(act, partials_ok=True)
+
+
+@register("feed_forward", "polynorm")
+class PolyNormFeedForward(Part):
+    """down(act(up x + b_up)) + b_down with act(z) = a N(z) + b N(z^2) + c N(z^3) + e, powers element by element,
+    N the division of a row of the hidden layer by its root mean square (eps inside the root).
+    params: hidden_size, intermediate_size, eps.  The four numbers are a tensor of the checkpoint."""
+
+    graph_safe = True  # launches depend on shapes only, never on the values of a step
+
+    @classmethod
+    def declare_weights(cls, params):
+        h, i = params["hidden_size"], params["intermediate_size"]
+        return {"up": WeightDecl((i, h)), "up_bias": WeightDecl((i,), init="zeros"), "down": WeightDecl((h, i)),
+                "down_bias": WeightDecl((h,), init="zeros"), "coef": WeightDecl((4,), init="ones")}
+
+    def __init__(self, params, tensors, rt, children=None):
+        super().__init__(params, tensors, rt, children)
+        self.eps = float(params["eps"])
+        self.up = Linear(tensors["up"], rt.weight_tiles)
+        self.down = Linear(tensors["down"], rt.weight_tiles)
+        self.up_bias, self.down_bias, self.coef = tensors["up_bias"], tensors["down_bias"], tensors["coef"]
+
+    def products(self):
+        if self.up.weight.dtype != torch.bfloat16:
+            return []
+        return [("up", self.up.out_features, self.up.in_features, False, None),
+                ("down", self.down.out_features, self.down.in_features, False, "norm")]
+
+    def forward(self, x):
+        """x [T, H] -> (delta, bias of the down projection): the block's next norm adds both."""
+        act = ops.polynorm(self.up(x), self.coef, self.eps, bias=self.up_bias)
+        return self.down(act, partials_ok=True), self.down_bias
