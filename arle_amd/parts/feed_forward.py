@@ -89,4 +89,5 @@ class PolyNormFeedForward(Part):
     def forward(self, x):
         """x [T, H] -> (delta, bias of the down projection): the block's next norm adds both."""
         act = ops.polynorm(self.up(x), self.coef, self.eps, bias=self.up_bias)
-        return self.down(act, partials_ok=True), self.down_bias
+        # float32 out: the sum goes into the 32-bit residual unrounded
+        return self.down(act, out_dtype=torch.float32, partials_ok=True), self.down_bias

@@ -79,4 +79,4 @@ class MLSTMMixer(Part):
                            cache["m"].state, batch.seg_row0, batch.seg_slot, heads=self.H, key_dim=self.D,
                            value_dim=self.Dv)
         y = ops.mlstm_output(o, g, self.norm, self.eps, self.rt.act_dtype, heads=self.H, value_dim=self.Dv)
-        return self.o(y, partials_ok=True)
+        return self.o(y, out_dtype=torch.float32, partials_ok=True)   # it goes into the 32-bit residual unrounded

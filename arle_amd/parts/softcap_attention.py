@@ -147,7 +147,7 @@ class SoftcapAttention(Part):
         softcap_attention(q, out, kv, batch, num_q_heads=self.nq, num_kv_heads=self.nkv, key_dim=self.Dk,
                           value_dim=self.Dv, scale=self.scale, softcap=self.softcap, r1=self.r1, r2=self.r2,
                           window=self.window or 0)
-        return self.o(out, partials_ok=True)
+        return self.o(out, out_dtype=torch.float32, partials_ok=True)   # it goes into the 32-bit residual unrounded
 
 
 def softcap_attention(q, out, kv, batch, *, num_q_heads, num_kv_heads, key_dim, value_dim, scale, softcap, r1, r2,
