@@ -70,8 +70,8 @@ class PolyNormFeedForward(Part):
     @classmethod
     def declare_weights(cls, params):
         h, i = params["hidden_size"], params["intermediate_size"]
-        return {"up": WeightDecl((i, h)), "up_bias": WeightDecl((i,), init="zeros"), "down": WeightDecl((h, i)),
-                "down_bias": WeightDecl((h,), init="zeros"), "coef": WeightDecl((4,), init="ones")}
+        return {"up": WeightDecl((i, h)), "up_bias": WeightDecl((i,), init="normal"), "down": WeightDecl((h, i)),
+                "down_bias": WeightDecl((h,), init="normal"), "coef": WeightDecl((4,), init="ones")}
 
     def __init__(self, params, tensors, rt, children=None):
         super().__init__(params, tensors, rt, children)

@@ -34,8 +34,8 @@ class MLSTMMixer(Part):
         w, h, d, dv = params["hidden_size"], params["heads"], params["key_dim"], params["value_dim"]
         return {"q": WeightDecl((h * d, w)), "k": WeightDecl((h * d, w)), "v": WeightDecl((h * dv, w)),
                 "g": WeightDecl((h * dv, w)), "o": WeightDecl((w, h * dv)), "norm": WeightDecl((h * dv,), init="ones"),
-                "i": WeightDecl((h, w)), "i_bias": WeightDecl((h,), init="zeros"),
-                "f": WeightDecl((h, w)), "f_bias": WeightDecl((h,), init="zeros")}
+                "i": WeightDecl((h, w)), "i_bias": WeightDecl((h,), init="normal"),
+                "f": WeightDecl((h, w)), "f_bias": WeightDecl((h,), init="normal")}
 
     @classmethod
     def declare_cache(cls, params):

@@ -52,7 +52,7 @@ class SoftcapAttention(Part):
             names += [("k", kw), ("v", vw)]
         for name, width in names:
             if params.get("bias"):
-                decl[name + "_bias"] = WeightDecl((width,), init="zeros")
+                decl[name + "_bias"] = WeightDecl((width,), init="normal")
             if taps:
                 decl[name + "_conv"] = WeightDecl((width, taps))
         if params.get("qk_norm"):

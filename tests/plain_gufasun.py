@@ -48,8 +48,9 @@ def attention_keys_values(h, p, m, eps):
     """Keys (after convolution and norm) and values (after convolution) of one layer for h [T, W]."""
     G, D, Dv = m["kv_heads"], m["dim"], m["vdim"]
     T = h.shape[0]
-    k = causal_conv(h @ p["k"].T + p["k.b"], p["k.conv"])
-    v = causal_conv(h @ p["v"].T + p["v.b"], p["v.conv"])
+    k, v = h @ p["k"].T + p["k.b"], h @ p["v"].T + p["v.b"]
+    if m.get("conv"):
+        k, v = causal_conv(k, p["k.conv"]), causal_conv(v, p["v.conv"])
     k = rms_unit(k.view(T, G, D), eps) * p["k.norm"]
     return k, v.view(T, G, Dv)
 
@@ -58,7 +59,9 @@ def attention_mixer(h, p, m, eps, keys, values):
     """Windowed soft-capped attention with a logarithmic distance penalty; keys [T, G, D], values [T, G, Dv]."""
     H, G, D = m["heads"], m["kv_heads"], m["dim"]
     T = h.shape[0]
-    q = causal_conv(h @ p["q"].T + p["q.b"], p["q.conv"])
+    q = h @ p["q"].T + p["q.b"]
+    if m.get("conv"):
+        q = causal_conv(q, p["q.conv"])
     q = rms_unit(q.view(T, H, D), eps) * p["q.norm"]
     pos = torch.arange(T, dtype=h.dtype)
     temp = 1 + m["q_temp"]["coef"] * torch.log(torch.floor((pos + 1) / m["q_temp"]["every"]) + 1)
