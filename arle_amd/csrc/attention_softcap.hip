@@ -201,3 +201,233 @@ extern "C" int arle_attn_softcap_simt(const void* q, long long q_stride, void* o
   }
   return launch_status();
 }
+
+// ---- matrix-core kernel (bfloat16) ------------------------------------------------------------
+// One wave a work item of sixteen queries that share a kv head: sixteen consecutive rows of one request for one
+// q head (prompt portions), or one decoded row for the up to sixteen q heads of a kv head.  The scores are
+// computed transposed, S^T[key][query] = K . Q^T with `v_mfma_f32_16x16x32_bf16`, so that a lane holds, for its
+// query (lane % 16), the keys 4g..4g+3 (g = lane / 16) of each sixteen-key half of a tile of 32 keys: the cap, the
+// penalty, the mask and the running softmax are per-lane arithmetic plus two lane exchanges, and the eight
+// probabilities of a lane are, as they lie, the B operand of the second product O^T += V^T . P^T once the keys of
+// the tile are taken in the order (4g..4g+3 of the first half, 4g..4g+3 of the second) on the V side too, which is
+// two 8-byte loads from the d-major value pages.  A half tile is sixteen slots of one page (page sizes are
+// multiples of 16).  Pages that a window has passed (entry -1) and slots beyond the newest key are never visible;
+// their keys are masked by a select and their values replaced by zeros, so that stale bits cannot reach a sum.
+namespace arle {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float fast_tanh(float x) { return 1.0f - 2.0f / (1.0f + __expf(2.0f * x)); }
+
+struct CapArgs {
+  const bf16* q; long long q_stride;
+  bf16* out; long long o_stride;
+  const bf16* k_pages; const bf16* v_pages;
+  const int* block_table; int table_stride;
+  const int* seg_row0; const int* seg_slot; const int* seg_start;
+  int segments, nq, nkv, Dk, Dv, page_size;
+  float scale, cap;
+  const void* r1; const void* r2; int r_dtype;
+  int window;
+};
+
+// KC: chunks of 32 of the key size held (Dk <= 32 KC); VC: chunks of 16 of the value size (Dv <= 16 VC).
+// HEADS: a work item is one row (a segment of one row) and the q heads of a kv head; else sixteen rows, one q head.
+template <int KC, int VC, bool HEADS>
+__global__ __launch_bounds__(kWave) void attn_softcap_mfma_kernel(const CapArgs a) {
+  const int lane = threadIdx.x, n = lane % 16, g = lane / 16;
+  const int group = a.nq / a.nkv;
+  int seg, row, head, kvh, first_row, last_row;
+  bool live;
+  if (HEADS) {
+    seg = blockIdx.x;
+    kvh = blockIdx.y;
+    row = first_row = last_row = a.seg_row0[seg];
+    head = kvh * group + min(n, group - 1);
+    live = n < group;
+  } else {
+    // the blockIdx.x-th block of sixteen rows, counted through the segments
+    int left = blockIdx.x, found = -1;
+    for (int s = 0; s < a.segments; ++s) {
+      const int blocks = (a.seg_row0[s + 1] - a.seg_row0[s] + 15) / 16;
+      if (left < blocks) {
+        found = s;
+        break;
+      }
+      left -= blocks;
+    }
+    if (found < 0) return;
+    seg = found;
+    head = blockIdx.y;
+    kvh = head / group;
+    const int end = a.seg_row0[seg + 1];
+    first_row = a.seg_row0[seg] + left * 16;
+    last_row = min(first_row + 15, end - 1);
+    live = first_row + n < end;
+    row = min(first_row + n, end - 1);
+  }
+  const int seg_first = a.seg_row0[seg];
+  const int pos = a.seg_start[seg] + (row - seg_first);
+  // keys that any query of the item sees: from the first row's window to the last row's own position
+  const int pos_lo = a.seg_start[seg] + (first_row - seg_first);
+  const int pos_hi = a.seg_start[seg] + (last_row - seg_first);
+  const int key_lo = a.window > 0 ? max(0, pos_lo - a.window + 1) : 0;
+  const int my_lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
+  const float pen1 = a.r1 ? load_as_float(a.r1, a.r_dtype, head) : 0.f;
+  const float pen2 = a.r1 ? load_as_float(a.r2, a.r_dtype, head) : 0.f;
+  const float inv_cap = a.cap > 0.f ? 1.0f / a.cap : 0.f;
+  const int n_kc = (a.Dk + 31) / 32, n_vc = a.Dv / 16;
+
+  // Q^T operand: for chunk c, Q[row][32 c + 8 g .. + 7]
+  bf16x8_t qreg[KC];
+  const bf16* qr = a.q + static_cast<int64_t>(row) * a.q_stride + head * a.Dk;
+#pragma unroll
+  for (int c = 0; c < KC; ++c) {
+    u32x4_t raw = {0, 0, 0, 0};
+    if (c < n_kc && 32 * c + 8 * g < a.Dk) raw = *reinterpret_cast<const u32x4_t*>(qr + 32 * c + 8 * g);
+    qreg[c] = __builtin_bit_cast(bf16x8_t, raw);
+  }
+  f32x4_t acc[VC];
+#pragma unroll
+  for (int c = 0; c < VC; ++c) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const int64_t k_page = static_cast<int64_t>(a.nkv) * a.page_size * a.Dk, v_page = static_cast<int64_t>(a.nkv) * a.page_size * a.Dv;
+  const int64_t k_head = static_cast<int64_t>(kvh) * a.page_size * a.Dk, v_head = static_cast<int64_t>(kvh) * a.page_size * a.Dv;
+
+  for (int tile = key_lo / 32; tile * 32 <= pos_hi; ++tile) {
+    const int key0 = tile * 32;
+    float s[8];
+    int page[2], in_page[2];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int kb = key0 + 16 * half;
+      const int entry = table[min(kb / a.page_size, a.table_stride - 1)];
+      page[half] = max(entry, 0);
+      in_page[half] = kb % a.page_size;
+      // S^T half tile: A = K[key kb + n][32 c + 8 g ..], B = Q^T
+      const bf16* kr = a.k_pages + page[half] * k_page + k_head + static_cast<int64_t>(in_page[half] + n) * a.Dk;
+      f32x4_t z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        if (c < n_kc) {
+          u32x4_t raw = {0, 0, 0, 0};
+          if (32 * c + 8 * g < a.Dk) raw = *reinterpret_cast<const u32x4_t*>(kr + 32 * c + 8 * g);
+          z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, raw), qreg[c], z, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb + 4 * g + i;
+        float v = z[i] * a.scale;
+        if (a.cap > 0.f) v = a.cap * fast_tanh(v * inv_cap);
+        if (a.r1) v -= pen1 * __logf(1.0f + pen2 * static_cast<float>(pos - key));
+        s[4 * half + i] = (key >= my_lo && key <= pos) ? v : -INFINITY;
+      }
+    }
+    float m_new = m_run;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m_new = fmaxf(m_new, s[i]);
+    m_new = fmaxf(m_new, __shfl_xor(m_new, 16, kWave));
+    m_new = fmaxf(m_new, __shfl_xor(m_new, 32, kWave));
+    // a query whose window begins behind this tile has seen nothing yet: keep its sums at zero without 0 * inf
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __expf(m_run - m_safe);
+    float p[8], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      p[i] = __expf(s[i] - m_safe);
+      sum += p[i];
+    }
+    sum += __shfl_xor(sum, 16, kWave);
+    sum += __shfl_xor(sum, 32, kWave);
+    l_run = l_run * alpha + sum;
+    m_run = m_new;
+    u32x4_t pb;
+    pb[0] = pack_bf16x2(p[0], p[1]);
+    pb[1] = pack_bf16x2(p[2], p[3]);
+    pb[2] = pack_bf16x2(p[4], p[5]);
+    pb[3] = pack_bf16x2(p[6], p[7]);
+    const bf16x8_t pop = __builtin_bit_cast(bf16x8_t, pb);
+    // which of this lane's eight key slots hold written keys (those between the item's first and last key)
+    const bool edge = key0 < key_lo || key0 + 31 > pos_hi;
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+      if (c < n_vc) {
+        u32x4_t vraw;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const bf16* vr = a.v_pages + page[half] * v_page + v_head + static_cast<int64_t>(16 * c + n) * a.page_size +
+                           in_page[half] + 4 * g;
+          const u32x2_t two = *reinterpret_cast<const u32x2_t*>(vr);
+          vraw[2 * half] = two[0];
+          vraw[2 * half + 1] = two[1];
+        }
+        if (edge) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int key = key0 + 16 * (j / 4) + 4 * g + j % 4;
+            if (key < key_lo || key > pos_hi) vraw[j / 2] &= (j % 2) ? 0x0000ffffu : 0xffff0000u;
+          }
+        }
+        f32x4_t o = acc[c];
+        o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+        acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vraw), pop, o, 0, 0, 0);
+      }
+    }
+  }
+  if (!live) return;
+  const float inv_l = 1.0f / l_run;
+  bf16* orow = a.out + static_cast<int64_t>(row) * a.o_stride + head * a.Dv;
+#pragma unroll
+  for (int c = 0; c < VC; ++c) {
+    if (c < n_vc) {
+      u32x2_t packed;
+      packed[0] = pack_bf16x2(acc[c][0] * inv_l, acc[c][1] * inv_l);
+      packed[1] = pack_bf16x2(acc[c][2] * inv_l, acc[c][3] * inv_l);
+      *reinterpret_cast<u32x2_t*>(orow + 16 * c + 4 * g) = packed;
+    }
+  }
+}
+
+}  // namespace arle
+
+// bfloat16 only.  Dk a multiple of 8 up to 256, Dv a multiple of 16 up to 256, page_size a multiple of 16, rows of
+// q and out 16-byte aligned (strides multiples of 8).  heads_mode: every segment is one row and nq / nkv <= 16.
+// row_blocks: an upper bound of the sixteen-row blocks of all segments (blocks past the last one return).
+extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* out, long long o_stride,
+                                      const void* k_pages, const void* v_pages, const int* block_table,
+                                      int table_stride, const int* seg_row0, const int* seg_slot, const int* seg_start,
+                                      int segments, int row_blocks, int heads_mode, int nq, int nkv, int Dk, int Dv,
+                                      int page_size, float scale, float cap, const void* r1, const void* r2,
+                                      int r_dtype, int window, void* stream) {
+  if (segments == 0) return 0;
+  if (Dk % 8 || Dk > 256 || Dv % 16 || Dv > 256 || page_size % 16 || nkv < 1 || nq % nkv || nq > 65535 ||
+      (heads_mode && nq / nkv > 16))
+    return static_cast<int>(hipErrorInvalidValue);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const CapArgs a{static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), o_stride,
+                  static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages), block_table, table_stride,
+                  seg_row0, seg_slot, seg_start, segments, nq, nkv, Dk, Dv, page_size, scale, cap, r1, r2, r_dtype, window};
+  const int size = (Dk + 1) / 2 > Dv ? (Dk + 1) / 2 : Dv;   // Dk counts half: a chunk of keys is 32 wide, of values 16
+#define ARLE_CAP(KC, VC)                                                                                \
+  do {                                                                                                  \
+    if (heads_mode)                                                                                     \
+      attn_softcap_mfma_kernel<KC, VC, true><<<dim3(segments, nkv), kWave, 0, s>>>(a);                  \
+    else                                                                                                \
+      attn_softcap_mfma_kernel<KC, VC, false><<<dim3(row_blocks, nq), kWave, 0, s>>>(a);                \
+  } while (0)
+  if (size <= 64) {
+    ARLE_CAP(4, 4);
+  } else if (size <= 128) {
+    ARLE_CAP(8, 8);
+  } else {
+    ARLE_CAP(8, 16);
+  }
+#undef ARLE_CAP
+  return launch_status();
+}

@@ -69,6 +69,8 @@ SIGNATURES = {
                                                   _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "arle_attn_softcap_simt": ("attention_softcap", [_p, _ll, _p, _ll, _p, _p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i,
                                                      _f, _f, _p, _p, _i, _i, _p]),
+    "arle_attn_softcap_mfma": ("attention_softcap", [_p, _ll, _p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i,
+                                                     _i, _f, _f, _p, _p, _i, _i, _p]),
     "arle_ceiling_read": ("ceilings", [_p, _ll, _i, _p, _p, _p]),
     "arle_ceiling_mfma": ("ceilings", [_i, _i, _i, _i, _p, _p]),
 }

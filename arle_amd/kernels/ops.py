@@ -1635,6 +1635,47 @@ def attn_softcap_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_
     return out
 
 
+CAP_MFMA_MAX_DIM = 256
+
+
 def attn_softcap_mfma_supported(dtype, key_dim: int, value_dim: int, page_size: int, group: int) -> bool:
     """Whether the matrix-core kernel of the soft-capped attention takes this shape."""
-    return False
+    return (dtype == torch.bfloat16 and key_dim % 8 == 0 and value_dim % 16 == 0 and page_size % 16 == 0
+            and key_dim <= CAP_MFMA_MAX_DIM and value_dim <= CAP_MFMA_MAX_DIM)
+
+
+def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *, max_qlen: int,
+                      num_q_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
+                      softcap: float = 0.0, r1=None, r2=None, window: int = 0):
+    """`attn_softcap_simt` on the matrix cores, bfloat16: sixteen rows of a segment a wave, or (when every segment is
+    one decoded row and a kv head has at most sixteen q heads) one row's q heads of a kv head a wave."""
+    _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, r1, r2)
+    tokens = q.shape[0]
+    _rows(q, "q")
+    _rows(out, "out")
+    group = num_q_heads // max(num_kv_heads, 1)
+    _need(attn_softcap_mfma_supported(q.dtype, key_dim, value_dim, page_size, group), "shape outside the matrix-core kernel's")
+    _need(q.shape == (tokens, num_q_heads * key_dim) and out.shape == (tokens, num_q_heads * value_dim)
+          and out.dtype == q.dtype, "q [T, nq*Dk] and out [T, nq*Dv] must be bfloat16")
+    _need(num_kv_heads > 0 and num_q_heads % num_kv_heads == 0 and num_q_heads <= _GRID_Y_MAX, "head counts out of range")
+    _need(q.stride(0) % 8 == 0 and out.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0,
+          "rows of q and out must be 16-byte aligned")
+    _check_kv_pages(k_pages, v_pages, num_kv_heads, page_size, key_dim, value_dim, q.dtype)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [slots, pages]")
+    segments = seg_slot.numel()
+    _i32(seg_slot, "seg_slot")
+    _i32(seg_start, "seg_start", segments)
+    _i32(seg_row0, "seg_row0", segments + 1)
+    _need((r1 is None) == (r2 is None), "give both distance constants or neither")
+    if r1 is not None:
+        _need(r1.shape == (num_q_heads,) and r2.shape == (num_q_heads,) and r1.dtype == r2.dtype and r1.dtype in _CODES
+              and r1.is_contiguous() and r2.is_contiguous(), "r1, r2 must be [heads] of one type")
+    heads_mode = max_qlen == 1 and group <= 16 and segments == tokens
+    row_blocks = tokens // 16 + segments      # no fewer than the sixteen-row blocks of all segments together
+    lib.call("arle_attn_softcap_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(),
+             v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], seg_row0.data_ptr(), seg_slot.data_ptr(),
+             seg_start.data_ptr(), segments, row_blocks, 1 if heads_mode else 0, num_q_heads, num_kv_heads, key_dim,
+             value_dim, page_size, float(scale), float(softcap), _ptr(r1), _ptr(r2),
+             _code(r1) if r1 is not None else 0, int(window), _stream())
+    return out
