@@ -220,7 +220,10 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ float fast_tanh(float x) { return 1.0f - 2.0f / (1.0f + __expf(2.0f * x)); }
+// tanh through one exponential and the hardware's reciprocal (a division in full would be a dozen instructions a score)
+__device__ __forceinline__ float fast_tanh(float x) {
+  return fmaf(-2.0f, __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * x)), 1.0f);
+}
 
 struct CapArgs {
   const bf16* q; long long q_stride;
@@ -235,10 +238,13 @@ struct CapArgs {
 };
 
 // KC: chunks of 32 of the key size held (Dk <= 32 KC); VC: chunks of 16 of the value size (Dv <= 16 VC).
-// HEADS: a work item is one row (a segment of one row) and the q heads of a kv head; else sixteen rows, one q head.
-template <int KC, int VC, bool HEADS>
-__global__ __launch_bounds__(kWave) void attn_softcap_mfma_kernel(const CapArgs a) {
-  const int lane = threadIdx.x, n = lane % 16, g = lane / 16;
+// HEADS: a work item is one row (a segment of one row) and the q heads of a kv head, and the WAVES waves of the
+// workgroup take its tiles of keys in turn and add their sums through LDS; else an item is sixteen rows of one q head,
+// and the waves of a workgroup are WAVES q heads of one kv head on the same rows, so that they fetch the same tiles.
+template <int KC, int VC, bool HEADS, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const CapArgs a) {
+  extern __shared__ float merge_lds[];   // HEADS: [WAVES][n_vc][64 lanes][4], then m [WAVES][16], l [WAVES][16]
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n = lane % 16, g = lane / 16;
   const int group = a.nq / a.nkv;
   int seg, row, head, kvh, first_row, last_row;
   bool live;
@@ -261,7 +267,7 @@ __global__ __launch_bounds__(kWave) void attn_softcap_mfma_kernel(const CapArgs 
     }
     if (found < 0) return;
     seg = found;
-    head = blockIdx.y;
+    head = blockIdx.y * WAVES + wave;
     kvh = head / group;
     const int end = a.seg_row0[seg + 1];
     first_row = a.seg_row0[seg] + left * 16;
@@ -298,31 +304,58 @@ __global__ __launch_bounds__(kWave) void attn_softcap_mfma_kernel(const CapArgs 
 
   const int64_t k_page = static_cast<int64_t>(a.nkv) * a.page_size * a.Dk, v_page = static_cast<int64_t>(a.nkv) * a.page_size * a.Dv;
   const int64_t k_head = static_cast<int64_t>(kvh) * a.page_size * a.Dk, v_head = static_cast<int64_t>(kvh) * a.page_size * a.Dv;
+  const int tile_step = HEADS ? WAVES : 1;
+  const int tile_first = key_lo / 32 + (HEADS ? wave : 0);
+  const int tile_last = pos_hi / 32, last_entry = a.table_stride - 1;
 
-  for (int tile = key_lo / 32; tile * 32 <= pos_hi; ++tile) {
-    const int key0 = tile * 32;
-    float s[8];
-    int page[2], in_page[2];
+  // Every load of a tile (K rows, V columns, after the two page ids) is sent a tile ahead, while the tile before it
+  // is worked through; a tile past the last is the last one again, fetched and dropped.
+  // The ids of the first 128 pages that the item sees are fetched once, a page a lane and two a lane, and read from
+  // there (a scalar lane read): a tile's loads then wait for no load of a page id before them.
+  const int page_first = key_lo / a.page_size;
+  const int held0 = table[min(page_first + lane, last_entry)], held1 = table[min(page_first + kWave + lane, last_entry)];
+  auto load_tile = [&](int tile, u32x4_t (&kraw)[2][KC], u32x4_t (&vraw)[VC]) {
+    const int key0 = min(tile, tile_last) * 32;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int kb = key0 + 16 * half;
-      const int entry = table[min(kb / a.page_size, a.table_stride - 1)];
-      page[half] = max(entry, 0);
-      in_page[half] = kb % a.page_size;
-      // S^T half tile: A = K[key kb + n][32 c + 8 g ..], B = Q^T
-      const bf16* kr = a.k_pages + page[half] * k_page + k_head + static_cast<int64_t>(in_page[half] + n) * a.Dk;
-      f32x4_t z = {0.f, 0.f, 0.f, 0.f};
+      const int rel = kb / a.page_size - page_first;
+      const int entry = rel < kWave         ? __builtin_amdgcn_readlane(held0, rel)
+                        : rel < 2 * kWave ? __builtin_amdgcn_readlane(held1, rel - kWave)
+                                          : table[min(kb / a.page_size, last_entry)];
+      const int64_t page = max(entry, 0);
+      const int in_page = kb % a.page_size;
+      const bf16* kr = a.k_pages + page * k_page + k_head + static_cast<int64_t>(in_page + n) * a.Dk;
 #pragma unroll
       for (int c = 0; c < KC; ++c) {
-        if (c < n_kc) {
-          u32x4_t raw = {0, 0, 0, 0};
-          if (32 * c + 8 * g < a.Dk) raw = *reinterpret_cast<const u32x4_t*>(kr + 32 * c + 8 * g);
-          z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, raw), qreg[c], z, 0, 0, 0);
-        }
+        kraw[half][c] = u32x4_t{0, 0, 0, 0};
+        if (c < n_kc && 32 * c + 8 * g < a.Dk) kraw[half][c] = *reinterpret_cast<const u32x4_t*>(kr + 32 * c + 8 * g);
       }
 #pragma unroll
+      for (int c = 0; c < VC; ++c) {
+        if (c < n_vc) {
+          const bf16* vr = a.v_pages + page * v_page + v_head + static_cast<int64_t>(16 * c + n) * a.page_size + in_page + 4 * g;
+          const u32x2_t two = *reinterpret_cast<const u32x2_t*>(vr);
+          vraw[c][2 * half] = two[0];
+          vraw[c][2 * half + 1] = two[1];
+        }
+      }
+    }
+  };
+
+  auto work_tile = [&](int tile, const u32x4_t (&kraw)[2][KC], const u32x4_t (&vraw)[VC]) {
+    const int key0 = tile * 32;
+    float s[8];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      // S^T half tile: A = K[key kb + n][32 c + 8 g ..], B = Q^T
+      f32x4_t z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < KC; ++c)
+        if (c < n_kc) z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kraw[half][c]), qreg[c], z, 0, 0, 0);
+#pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = kb + 4 * g + i;
+        const int key = key0 + 16 * half + 4 * g + i;
         float v = z[i] * a.scale;
         if (a.cap > 0.f) v = a.cap * fast_tanh(v * inv_cap);
         if (a.r1) v -= pen1 * __logf(1.0f + pen2 * static_cast<float>(pos - key));
@@ -358,27 +391,80 @@ __global__ __launch_bounds__(kWave) void attn_softcap_mfma_kernel(const CapArgs 
 #pragma unroll
     for (int c = 0; c < VC; ++c) {
       if (c < n_vc) {
-        u32x4_t vraw;
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const bf16* vr = a.v_pages + page[half] * v_page + v_head + static_cast<int64_t>(16 * c + n) * a.page_size +
-                           in_page[half] + 4 * g;
-          const u32x2_t two = *reinterpret_cast<const u32x2_t*>(vr);
-          vraw[2 * half] = two[0];
-          vraw[2 * half + 1] = two[1];
-        }
+        u32x4_t vr = vraw[c];
         if (edge) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const int key = key0 + 16 * (j / 4) + 4 * g + j % 4;
-            if (key < key_lo || key > pos_hi) vraw[j / 2] &= (j % 2) ? 0x0000ffffu : 0xffff0000u;
+            if (key < key_lo || key > pos_hi) vr[j / 2] &= (j % 2) ? 0x0000ffffu : 0xffff0000u;
           }
         }
         f32x4_t o = acc[c];
         o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
-        acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vraw), pop, o, 0, 0, 0);
+        acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vr), pop, o, 0, 0, 0);
       }
     }
+  };
+
+  if (HEADS) {
+    // a decoded row's waves are few and each walks a chain of tiles: the next tile's loads fly while this one is worked
+    u32x4_t k_even[2][KC], v_even[VC], k_odd[2][KC], v_odd[VC];
+    if (tile_first <= tile_last) load_tile(tile_first, k_even, v_even);
+    for (int tile = tile_first; tile <= tile_last; tile += 2 * tile_step) {
+      load_tile(tile + tile_step, k_odd, v_odd);
+      work_tile(tile, k_even, v_even);
+      if (tile + tile_step > tile_last) break;
+      load_tile(tile + 2 * tile_step, k_even, v_even);
+      work_tile(tile + tile_step, k_odd, v_odd);
+    }
+  } else {
+    // portions bring thousands of waves: more of them a SIMD hide the loads better than a second set of registers
+    // (measured: 2,048 rows behind a window of 1,024, 256 us a layer this way, 388 with the tile fetched ahead)
+    u32x4_t k_now[2][KC], v_now[VC];
+    for (int tile = tile_first; tile <= tile_last; ++tile) {
+      load_tile(tile, k_now, v_now);
+      work_tile(tile, k_now, v_now);
+    }
+  }
+
+  if (HEADS && WAVES > 1) {
+    // the waves' sums meet in LDS; wave w then finishes the chunks w, w + WAVES, ... of the value size
+    f32x4_t* part = reinterpret_cast<f32x4_t*>(merge_lds);
+    float* part_m = merge_lds + WAVES * n_vc * kWave * 4;
+    float* part_l = part_m + WAVES * 16;
+#pragma unroll
+    for (int c = 0; c < VC; ++c)
+      if (c < n_vc) part[(wave * n_vc + c) * kWave + lane] = acc[c];
+    if (g == 0) {
+      part_m[wave * 16 + n] = m_run;
+      part_l[wave * 16 + n] = l_run;
+    }
+    __syncthreads();
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) m_all = fmaxf(m_all, part_m[w * 16 + n]);
+    float l_all = 0.f, f[WAVES];
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      f[w] = __expf(part_m[w * 16 + n] - m_all);
+      l_all += part_l[w * 16 + n] * f[w];
+    }
+    if (!live) return;
+    const float inv_l = 1.0f / l_all;
+    bf16* orow = a.out + static_cast<int64_t>(row) * a.o_stride + head * a.Dv;
+    for (int c = wave; c < n_vc; c += WAVES) {
+      f32x4_t o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) {
+        const f32x4_t t = part[(w * n_vc + c) * kWave + lane];
+        o[0] += t[0] * f[w]; o[1] += t[1] * f[w]; o[2] += t[2] * f[w]; o[3] += t[3] * f[w];
+      }
+      u32x2_t packed;
+      packed[0] = pack_bf16x2(o[0] * inv_l, o[1] * inv_l);
+      packed[1] = pack_bf16x2(o[2] * inv_l, o[3] * inv_l);
+      *reinterpret_cast<u32x2_t*>(orow + 16 * c + 4 * g) = packed;
+    }
+    return;
   }
   if (!live) return;
   const float inv_l = 1.0f / l_run;
@@ -393,6 +479,8 @@ __global__ __launch_bounds__(kWave) void attn_softcap_mfma_kernel(const CapArgs 
     }
   }
 }
+
+constexpr int kCapSplitWaves = 8;   // waves that share the keys of a decoded row
 
 }  // namespace arle
 
@@ -414,15 +502,34 @@ extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* o
                   static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages), block_table, table_stride,
                   seg_row0, seg_slot, seg_start, segments, nq, nkv, Dk, Dv, page_size, scale, cap, r1, r2, r_dtype, window};
   const int size = (Dk + 1) / 2 > Dv ? (Dk + 1) / 2 : Dv;   // Dk counts half: a chunk of keys is 32 wide, of values 16
-#define ARLE_CAP(KC, VC)                                                                                \
-  do {                                                                                                  \
-    if (heads_mode)                                                                                     \
-      attn_softcap_mfma_kernel<KC, VC, true><<<dim3(segments, nkv), kWave, 0, s>>>(a);                  \
-    else                                                                                                \
-      attn_softcap_mfma_kernel<KC, VC, false><<<dim3(row_blocks, nq), kWave, 0, s>>>(a);                \
+  const int group = nq / nkv;
+  const int head_waves = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);   // q heads of one kv head that share a workgroup
+  const size_t merge_bytes = static_cast<size_t>(kCapSplitWaves) * ((Dv / 16) * kWave * 4 + 32) * sizeof(float);
+#define ARLE_CAP(KC, VC)                                                                                           \
+  do {                                                                                                             \
+    if (heads_mode) {                                                                                              \
+      static bool raised = false;   /* more LDS than a launch gets unasked: said once for the kernel */            \
+      if (!raised && merge_bytes > 48 * 1024) {                                                                    \
+        const hipError_t e = hipFuncSetAttribute(                                                                  \
+            reinterpret_cast<const void*>(&attn_softcap_mfma_kernel<KC, VC, true, kCapSplitWaves>),                \
+            hipFuncAttributeMaxDynamicSharedMemorySize, kCapSplitWaves * (VC * kWave * 4 + 32) * 4);              \
+        if (e != hipSuccess) return static_cast<int>(e);                                                           \
+        raised = true;                                                                                             \
+      }                                                                                                            \
+      attn_softcap_mfma_kernel<KC, VC, true, kCapSplitWaves>                                                       \
+          <<<dim3(segments, nkv), kCapSplitWaves * kWave, merge_bytes, s>>>(a);                                    \
+    }                                                                                                              \
+    else if (head_waves == 4)                                                                                      \
+      attn_softcap_mfma_kernel<KC, VC, false, 4><<<dim3(row_blocks, nq / 4), 4 * kWave, 0, s>>>(a);                \
+    else if (head_waves == 2)                                                                                      \
+      attn_softcap_mfma_kernel<KC, VC, false, 2><<<dim3(row_blocks, nq / 2), 2 * kWave, 0, s>>>(a);                \
+    else                                                                                                           \
+      attn_softcap_mfma_kernel<KC, VC, false, 1><<<dim3(row_blocks, nq), kWave, 0, s>>>(a);                        \
   } while (0)
   if (size <= 64) {
     ARLE_CAP(4, 4);
+  } else if (Dk <= 128 && Dv <= 128) {
+    ARLE_CAP(4, 8);
   } else if (size <= 128) {
     ARLE_CAP(8, 8);
   } else {

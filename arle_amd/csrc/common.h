@@ -102,6 +102,34 @@ __device__ __forceinline__ void store_from_float(void* p, int code, int64_t i, f
   }
 }
 
+// Four consecutive elements as floats, by one 16-byte (float) or 8-byte (bfloat16) access; the address is aligned
+// to that size.
+template <typename T>
+__device__ __forceinline__ float4 ld4(const T* p);
+template <>
+__device__ __forceinline__ float4 ld4<float>(const float* p) {
+  return *reinterpret_cast<const float4*>(p);
+}
+template <>
+__device__ __forceinline__ float4 ld4<bf16>(const bf16* p) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  return float4{__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                __uint_as_float(raw.y & 0xffff0000u)};
+}
+template <typename T>
+__device__ __forceinline__ void st4(T* p, float4 v);
+template <>
+__device__ __forceinline__ void st4<float>(float* p, float4 v) {
+  *reinterpret_cast<float4*>(p) = v;
+}
+template <>
+__device__ __forceinline__ void st4<bf16>(bf16* p, float4 v) {
+  uint2 raw;
+  raw.x = pack_bf16x2(v.x, v.y);
+  raw.y = pack_bf16x2(v.z, v.w);
+  *reinterpret_cast<uint2*>(p) = raw;
+}
+
 inline int launch_status() { return static_cast<int>(hipGetLastError()); }
 
 // Element type codes shared with the Python side.

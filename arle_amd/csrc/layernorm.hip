@@ -83,6 +83,123 @@ __global__ __launch_bounds__(kLnThreads) void add_layernorm_kernel(
   }
 }
 
+// The same for the usual types: terms that are float32 (a projection's 32-bit output or its stack of partial
+// products), biases, weights and outputs of one type TA, a width that is a multiple of 4.  Four elements a lane and
+// access, every load of a row issued without a condition on data, before anything is stored.
+template <typename TA, int PER4>
+__global__ __launch_bounds__(kLnThreads) void add_layernorm_vec_kernel(
+    float* __restrict__ residual, const float* __restrict__ t0, int n0, long long s0, const TA* __restrict__ b0,
+    const float* __restrict__ t1, int n1, long long s1, const TA* __restrict__ b1, const TA* __restrict__ wa,
+    const TA* __restrict__ wb, TA* __restrict__ out_a, TA* __restrict__ out_b, const int* __restrict__ rows, int width,
+    float eps) {
+  __shared__ float lds[kLnWaves];
+  const int r = blockIdx.x;
+  const int64_t src = rows ? rows[r] : r;
+  const int64_t base = src * width;
+  const int last = width - 4, tid = threadIdx.x;
+  float4 x[PER4];
+#pragma unroll
+  for (int k = 0; k < PER4; ++k) x[k] = ld4<float>(residual + base + min((tid + k * kLnThreads) * 4, last));
+  auto add_term = [&](const float* t, int n, long long stride, const TA* bias) {
+    float4 d[PER4];
+#pragma unroll
+    for (int k = 0; k < PER4; ++k) d[k] = ld4<float>(t + base + min((tid + k * kLnThreads) * 4, last));
+    // the parts of a stack are fetched several at a time (eight for rows up to 4,096 wide) without a condition (a part past the last is the last one
+    // again, fetched and dropped), so that their loads are in flight together; they are added in the stack's order
+    constexpr int G = PER4 <= 4 ? 8 : (PER4 <= 8 ? 4 : 2);
+    for (int s0 = 1; s0 < n; s0 += G) {
+      float4 e[G][PER4];
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const long long at = min(s0 + j, n - 1) * stride + base;
+#pragma unroll
+        for (int k = 0; k < PER4; ++k) e[j][k] = ld4<float>(t + at + min((tid + k * kLnThreads) * 4, last));
+      }
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        if (s0 + j < n) {
+#pragma unroll
+          for (int k = 0; k < PER4; ++k) {
+            d[k].x += e[j][k].x; d[k].y += e[j][k].y; d[k].z += e[j][k].z; d[k].w += e[j][k].w;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < PER4; ++k) {
+      if (bias) {
+        const float4 e = ld4<TA>(bias + min((tid + k * kLnThreads) * 4, last));
+        d[k].x += e.x; d[k].y += e.y; d[k].z += e.z; d[k].w += e.w;
+      }
+      x[k].x += d[k].x; x[k].y += d[k].y; x[k].z += d[k].z; x[k].w += d[k].w;
+    }
+  };
+  // the norm weights are fetched now, not behind the two reductions that their use waits for
+  float4 w_a[PER4], w_b[PER4];
+#pragma unroll
+  for (int k = 0; k < PER4; ++k) {
+    w_a[k] = ld4<TA>(wa + min((tid + k * kLnThreads) * 4, last));
+    w_b[k] = ld4<TA>((wb ? wb : wa) + min((tid + k * kLnThreads) * 4, last));
+  }
+  if (t0) add_term(t0, n0, s0, b0);
+  if (t1) add_term(t1, n1, s1, b1);
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < PER4; ++k) {
+    const int i = (tid + k * kLnThreads) * 4;
+    if (i < width) {
+      if (!rows && (t0 || t1)) st4<float>(residual + base + i, x[k]);
+      sum += (x[k].x + x[k].y) + (x[k].z + x[k].w);
+    }
+  }
+  const float mu = block_sum<kLnWaves>(sum, lds) / static_cast<float>(width);
+  float sq = 0.f;
+#pragma unroll
+  for (int k = 0; k < PER4; ++k) {
+    const int i = (tid + k * kLnThreads) * 4;
+    x[k].x -= mu; x[k].y -= mu; x[k].z -= mu; x[k].w -= mu;
+    if (i < width) sq += (x[k].x * x[k].x + x[k].y * x[k].y) + (x[k].z * x[k].z + x[k].w * x[k].w);
+  }
+  const float inv = 1.0f / sqrtf(block_sum<kLnWaves>(sq, lds) / static_cast<float>(width) + eps);
+  const int64_t o = static_cast<int64_t>(r) * width;
+#pragma unroll
+  for (int k = 0; k < PER4; ++k) {
+    const int i = (tid + k * kLnThreads) * 4;
+    if (i < width) {
+      const float4 w = w_a[k];
+      st4<TA>(out_a + o + i, float4{x[k].x * inv * w.x, x[k].y * inv * w.y, x[k].z * inv * w.z, x[k].w * inv * w.w});
+      if (out_b) {
+        const float4 v = w_b[k];
+        st4<TA>(out_b + o + i, float4{x[k].x * inv * v.x, x[k].y * inv * v.y, x[k].z * inv * v.z, x[k].w * inv * v.w});
+      }
+    }
+  }
+}
+
+template <typename TA>
+static int launch_ln_vec(float* residual, const LnTerm& t0, const LnTerm& t1, const void* wa, const void* wb, void* out_a,
+                         void* out_b, const int* rows, int n_rows, int width, float eps, hipStream_t s) {
+#define ARLE_LNV(PER4)                                                                                              \
+  add_layernorm_vec_kernel<TA, PER4><<<n_rows, kLnThreads, 0, s>>>(                                                  \
+      residual, static_cast<const float*>(t0.data), t0.n_stack, t0.stack_stride, static_cast<const TA*>(t0.bias),  \
+      static_cast<const float*>(t1.data), t1.n_stack, t1.stack_stride, static_cast<const TA*>(t1.bias),            \
+      static_cast<const TA*>(wa), static_cast<const TA*>(wb), static_cast<TA*>(out_a), static_cast<TA*>(out_b), rows, \
+      width, eps)
+  if (width <= kLnThreads * 4) {
+    ARLE_LNV(1);
+  } else if (width <= kLnThreads * 8) {
+    ARLE_LNV(2);
+  } else if (width <= kLnThreads * 16) {
+    ARLE_LNV(4);
+  } else if (width <= kLnThreads * 32) {
+    ARLE_LNV(8);
+  } else {
+    ARLE_LNV(16);
+  }
+#undef ARLE_LNV
+  return launch_status();
+}
+
 }  // namespace arle
 
 using namespace arle;
@@ -99,6 +216,12 @@ extern "C" int arle_add_layernorm(float* residual, const void* term0, int n0, lo
   hipStream_t s = static_cast<hipStream_t>(stream);
   const LnTerm t0{term0, n0, stride0, dtype0, bias0, bias_dtype0};
   const LnTerm t1{term1, n1, stride1, dtype1, bias1, bias_dtype1};
+  // the usual case: float32 terms, everything else of the output's type, whole groups of four
+  const auto fits = [&](const LnTerm& t) { return !t.data || (t.dtype == kF32 && (!t.bias || t.bias_dtype == out_dtype)); };
+  if (width % 4 == 0 && fits(t0) && fits(t1) && w_dtype == out_dtype) {
+    return out_dtype == kF32 ? launch_ln_vec<float>(residual, t0, t1, wa, wb, out_a, out_b, rows, n_rows, width, eps, s)
+                             : launch_ln_vec<bf16>(residual, t0, t1, wa, wb, out_a, out_b, rows, n_rows, width, eps, s);
+  }
 #define ARLE_LN(PER)                                                                                          \
   add_layernorm_kernel<PER><<<n_rows, kLnThreads, 0, s>>>(residual, t0, t1, wa, wb, w_dtype, out_a, out_b, \
                                                           out_dtype, rows, width, eps)

@@ -47,6 +47,53 @@ __global__ void causal_conv_kernel(const void* __restrict__ u, long long u_strid
   store_from_float(out, out_dtype, t * out_stride + c, acc);
 }
 
+// One element type T throughout and channels in whole groups of four: a lane takes four channels of a row with one
+// access each for the input, the taps - 1 rows before it (the step's, or the state's) and the weights; none of the
+// loads stands under a condition on data (which rows are the step's is the same for the whole workgroup).
+template <typename T, int TAPS>
+__global__ void causal_conv_vec_kernel(const T* __restrict__ u, long long u_stride, const T* __restrict__ bias,
+                                       const T* __restrict__ w, const T* __restrict__ state,
+                                       const int* __restrict__ slot_of_token, T* __restrict__ out, long long out_stride,
+                                       int channels, int add_input) {
+  const int t = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
+  if (c >= channels) return;
+  const int slot = slot_of_token[t];
+  int mine = 0;
+  while (mine < TAPS - 1 && t - mine - 1 >= 0 && slot_of_token[t - mine - 1] == slot) ++mine;
+  const float4 b = bias ? ld4<T>(bias + c) : float4{0.f, 0.f, 0.f, 0.f};
+  float4 in[TAPS];     // in[back]: the input `back` rows before this one
+#pragma unroll
+  for (int back = 0; back < TAPS; ++back) {
+    if (back <= mine) {
+      const float4 v = ld4<T>(u + (t - back) * u_stride + c);
+      in[back] = float4{v.x + b.x, v.y + b.y, v.z + b.z, v.w + b.w};
+    } else {
+      const int64_t row = static_cast<int64_t>(slot) * (TAPS - 1) + (TAPS - 1 - (back - mine));
+      in[back] = ld4<T>(state + row * channels + c);
+    }
+  }
+  float wt[4][TAPS];   // four channels' taps are 4 * TAPS consecutive elements
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) {
+    const float4 v = ld4<T>(w + static_cast<int64_t>(c) * TAPS + 4 * j);
+    const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wt[(4 * j + i) / TAPS][(4 * j + i) % TAPS] = e[i];
+  }
+  float acc[4];
+  const float now[4] = {in[0].x, in[0].y, in[0].z, in[0].w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = fmaf(wt[i][TAPS - 1], now[i], add_input ? now[i] : 0.f);
+#pragma unroll
+  for (int back = 1; back < TAPS; ++back) {
+    const float v[4] = {in[back].x, in[back].y, in[back].z, in[back].w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = fmaf(wt[i][TAPS - 1 - back], v[i], acc[i]);
+  }
+  st4<T>(out + t * out_stride + c, float4{acc[0], acc[1], acc[2], acc[3]});
+}
+
 // One thread a (segment, channel): the new state is the last taps-1 of (old state, this step's inputs).
 __global__ void conv_state_update_kernel(const void* __restrict__ u, long long u_stride, int u_dtype,
                                          const void* __restrict__ bias, int bias_dtype, void* __restrict__ state,
@@ -85,6 +132,25 @@ extern "C" int arle_causal_conv(const void* u, long long u_stride, int u_dtype, 
                                 int channels, int taps, int add_input, void* stream) {
   if (tokens == 0 || channels == 0) return 0;
   if (w && (taps < 1 || taps > kConvMaxTaps)) return static_cast<int>(hipErrorInvalidValue);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const auto at16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if (w && taps >= 2 && taps <= 4 && channels % 4 == 0 && u_stride % 4 == 0 && out_stride % 4 == 0 && at16(u) && at16(out) &&
+      at16(state) && u_dtype == out_dtype && w_dtype == out_dtype && state_dtype == out_dtype &&
+      (!bias || bias_dtype == out_dtype)) {
+    dim3 vgrid(tokens, (channels / 4 + 255) / 256);
+#define ARLE_CONV(T, TAPS)                                                                                          \
+  causal_conv_vec_kernel<T, TAPS><<<vgrid, 256, 0, s>>>(static_cast<const T*>(u), u_stride, static_cast<const T*>(bias), \
+                                                        static_cast<const T*>(w), static_cast<const T*>(state),       \
+                                                        slot_of_token, static_cast<T*>(out), out_stride, channels,    \
+                                                        add_input)
+    if (out_dtype == kF32) {
+      if (taps == 2) ARLE_CONV(float, 2); else if (taps == 3) ARLE_CONV(float, 3); else ARLE_CONV(float, 4);
+    } else {
+      if (taps == 2) ARLE_CONV(bf16, 2); else if (taps == 3) ARLE_CONV(bf16, 3); else ARLE_CONV(bf16, 4);
+    }
+#undef ARLE_CONV
+    return launch_status();
+  }
   dim3 grid(tokens, (channels + 255) / 256);
   causal_conv_kernel<<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(
       u, u_stride, u_dtype, bias, bias_dtype, w, w_dtype, state, state_dtype, slot_of_token, out, out_stride,

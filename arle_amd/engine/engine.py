@@ -213,8 +213,16 @@ class Engine:
         self.cache.append([(e.request, len(e.tokens)) for e in entries])
         saved_state = None
         try:
-            # a mixer with state of its own overwrites it while the step runs: keep what a failed step must leave
-            saved_state = self.cache.snapshot_state([e.request for e in entries])
+            # a mixer with state of its own overwrites it while the step runs: keep what a failed step must leave.
+            # A step that is replayed from its graph runs no Python between its kernels, so nothing can fail half way.
+            if decode_only:
+                rows_now = len(entries)
+                replayed = (rows_now, self.model.decode_launch_class(
+                    rows_now, max(before[e.request] for e in entries) + 1)) in self._graphs
+            else:
+                replayed = shape_key is not None and shape_key in self._graphs
+            if not replayed:
+                saved_state = self.cache.snapshot_state([e.request for e in entries])
             self.cache.sync_tables()
             if decode_only:
                 logits = self._decode_step_graphed(entries, before, borrow_logits)

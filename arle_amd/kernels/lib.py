@@ -62,9 +62,9 @@ SIGNATURES = {
     "arle_causal_conv": ("short_conv", [_p, _ll, _i, _p, _i, _p, _i, _p, _i, _p, _p, _ll, _i, _i, _i, _i, _i, _p]),
     "arle_conv_state_update": ("short_conv", [_p, _ll, _i, _p, _i, _p, _i, _p, _p, _i, _i, _i, _p]),
     "arle_polynorm": ("polynorm", [_p, _ll, _i, _p, _i, _p, _i, _p, _i, _i, _i, _f, _p]),
-    "arle_mlstm_scan": ("mlstm", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _ll, _p, _p, _i, _f, _p, _p, _p, _p, _p, _i, _p, _p,
+    "arle_mlstm_scan": ("mlstm", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _ll, _p, _p, _f, _p, _p, _p, _p, _p, _i, _p, _p, _p,
                                   _i, _i, _i, _p]),
-    "arle_mlstm_output": ("mlstm", [_p, _p, _ll, _i, _p, _i, _p, _i, _i, _i, _i, _f, _p]),
+    "arle_mlstm_output": ("mlstm", [_p, _p, _p, _p, _ll, _i, _p, _i, _p, _i, _i, _i, _i, _f, _p]),
     "arle_qkv_norm_store": ("attention_softcap", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _f, _f, _i, _p, _p, _p, _i,
                                                   _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "arle_attn_softcap_simt": ("attention_softcap", [_p, _ll, _p, _ll, _p, _p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i,

@@ -1512,9 +1512,10 @@ MLSTM_MAX_KEY_DIM = 256
 
 def mlstm_scan(q, k, v, gates, bias_i, bias_f, cap: float, s_state, n_state, m_state, seg_row0, seg_slot, *,
                heads: int, key_dim: int, value_dim: int):
-    """The matrix-memory recurrence over the rows of every segment, from and into the requests' states; returns
-    float32 [T, heads * value_dim]: S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6) with q scaled by
-    key_dim^(-1/2).  gates float32 [T, 2 * heads]: pre-activations of the input gates, then of the forget gates."""
+    """The matrix-memory recurrence over the rows of every segment, from and into the requests' states.  Returns
+    (num float32 [T, heads * value_dim], nq float32 [T, heads], coefs float32 [T, heads, 3]): the numerators
+    S_t^T q_t and n_t . q_t with q scaled by key_dim^(-1/2), and (keep, take, m_t) of every row and head, for
+    `mlstm_output`.  gates float32 [T, 2 * heads]: pre-activations of the input gates, then of the forget gates."""
     _gpu(q, k, v, gates, bias_i, bias_f, s_state, n_state, m_state, seg_row0, seg_slot)
     H, D, Dv = heads, key_dim, value_dim
     tokens = q.shape[0]
@@ -1524,8 +1525,8 @@ def mlstm_scan(q, k, v, gates, bias_i, bias_f, cap: float, s_state, n_state, m_s
     _need(0 < D <= MLSTM_MAX_KEY_DIM, f"the mLSTM kernels take key sizes up to {MLSTM_MAX_KEY_DIM}")
     _rows(gates, "gates")
     _need(gates.dtype == torch.float32 and gates.shape == (tokens, 2 * H), "gates must be float32 [T, 2 * heads]")
-    _need(bias_i.shape == (H,) and bias_f.shape == (H,) and bias_i.dtype == bias_f.dtype and bias_i.is_contiguous()
-          and bias_f.is_contiguous(), "gate biases must be [heads] of one type")
+    _need(bias_i.shape == (H,) and bias_f.shape == (H,) and bias_i.dtype == bias_f.dtype == torch.float32
+          and bias_i.is_contiguous() and bias_f.is_contiguous(), "gate biases must be float32 [heads]")
     slots = s_state.shape[0]
     _need(s_state.shape == (slots, H, D, Dv) and n_state.shape == (slots, H, D) and m_state.shape == (slots, H)
           and all(t.dtype == torch.float32 and t.is_contiguous() for t in (s_state, n_state, m_state)),
@@ -1534,26 +1535,32 @@ def mlstm_scan(q, k, v, gates, bias_i, bias_f, cap: float, s_state, n_state, m_s
     _i32(seg_slot, "seg_slot")
     _i32(seg_row0, "seg_row0", segments + 1)
     coefs = torch.empty((tokens, H, 3), dtype=torch.float32, device=q.device)
-    o = torch.empty((tokens, H * Dv), dtype=torch.float32, device=q.device)
+    num = torch.empty((tokens, H * Dv), dtype=torch.float32, device=q.device)
+    nq = torch.empty((tokens, H), dtype=torch.float32, device=q.device)
     lib.call("arle_mlstm_scan", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), _code(q),
-             gates.data_ptr(), gates.stride(0), bias_i.data_ptr(), bias_f.data_ptr(), _code(bias_i), float(cap),
+             gates.data_ptr(), gates.stride(0), bias_i.data_ptr(), bias_f.data_ptr(), float(cap),
              s_state.data_ptr(), n_state.data_ptr(), m_state.data_ptr(), seg_row0.data_ptr(), seg_slot.data_ptr(),
-             segments, coefs.data_ptr(), o.data_ptr(), H, D, Dv, _stream())
-    return o
+             segments, coefs.data_ptr(), num.data_ptr(), nq.data_ptr(), H, D, Dv, _stream())
+    return num, nq, coefs
 
 
-def mlstm_output(o, gate, weight, eps: float, out_dtype, *, heads: int, value_dim: int):
-    """Each head's o divided by its root mean square, times `weight` [heads * value_dim], times sigmoid(gate)."""
-    _gpu(o, gate, weight)
-    tokens = o.shape[0]
+def mlstm_output(num, nq, coefs, gate, weight, eps: float, out_dtype, *, heads: int, value_dim: int):
+    """o = num / (max(|nq|, exp(-m)) + 1e-6); then each head's o divided by its root mean square, times `weight`
+    [heads * value_dim], times sigmoid(gate)."""
+    _gpu(num, nq, coefs, gate, weight)
+    tokens = num.shape[0]
     width = heads * value_dim
-    _need(o.dtype == torch.float32 and o.shape == (tokens, width) and o.is_contiguous(), "o must be float32 [T, H * Dv]")
+    _need(num.dtype == torch.float32 and num.shape == (tokens, width) and num.is_contiguous(), "num must be float32 [T, H * Dv]")
+    _need(nq.dtype == torch.float32 and nq.shape == (tokens, heads) and nq.is_contiguous()
+          and coefs.dtype == torch.float32 and coefs.shape == (tokens, heads, 3) and coefs.is_contiguous(),
+          "nq [T, H] and coefs [T, H, 3] must be float32")
     _rows(gate, "gate")
     _need(gate.shape == (tokens, width) and gate.dtype in _CODES, "gate must be [T, H * Dv]")
     _need(weight.shape == (width,) and weight.is_contiguous() and weight.dtype in _CODES, "the norm weight must be [H * Dv]")
-    out = torch.empty((tokens, width), dtype=out_dtype, device=o.device)
-    lib.call("arle_mlstm_output", o.data_ptr(), gate.data_ptr(), gate.stride(0), _code(gate), weight.data_ptr(),
-             _code(weight), out.data_ptr(), _code(out), tokens, heads, value_dim, float(eps), _stream())
+    out = torch.empty((tokens, width), dtype=out_dtype, device=num.device)
+    lib.call("arle_mlstm_output", num.data_ptr(), nq.data_ptr(), coefs.data_ptr(), gate.data_ptr(), gate.stride(0),
+             _code(gate), weight.data_ptr(), _code(weight), out.data_ptr(), _code(out), tokens, heads, value_dim,
+             float(eps), _stream())
     return out
 
 

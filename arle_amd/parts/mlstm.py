@@ -57,8 +57,16 @@ class MLSTMMixer(Part):
         if len({t.dtype for t in fused}) != 1:
             raise ValueError("q, k, v and gate projections must be stored in one type")
         self.qkvg = Linear(torch.cat(fused, dim=0).contiguous(), rt.weight_tiles)
-        # the gates enter the recurrence: their projection is a 32-bit product whatever the mode
-        self.gates = torch.cat([tensors["i"], tensors["f"]], dim=0).float().contiguous()
+        # The gates enter the recurrence: their projection hands over 32-bit sums whatever the mode.  In bfloat16 it
+        # is a product of bfloat16 operands like every projection (rows padded with zeros to whole tiles of 16 outputs),
+        # in float32 the fixed-order 32-bit product.
+        gates = torch.cat([tensors["i"], tensors["f"]], dim=0)
+        if gates.dtype == torch.bfloat16 and not rt.is_f32:
+            pad = -gates.shape[0] % 16
+            gates = torch.cat([gates, gates.new_zeros((pad, gates.shape[1]))], dim=0) if pad else gates
+            self.gates = Linear(gates.contiguous(), rt.weight_tiles)
+        else:
+            self.gates = Linear(gates.float().contiguous())
         self.i_bias, self.f_bias = tensors["i_bias"].float().contiguous(), tensors["f_bias"].float().contiguous()
         self.norm = tensors["norm"]
         self.o = Linear(tensors["o"], rt.weight_tiles)
@@ -74,9 +82,9 @@ class MLSTMMixer(Part):
         qk, vw = self.H * self.D, self.H * self.Dv
         p = self.qkvg(x)
         q, k, v, g = p[:, :qk], p[:, qk:2 * qk], p[:, 2 * qk:2 * qk + vw], p[:, 2 * qk + vw:]
-        gates = ops.gemm_f32(x if x.dtype == torch.float32 else x.float(), self.gates)
-        o = ops.mlstm_scan(q, k, v, gates, self.i_bias, self.f_bias, self.cap, cache["S"].state, cache["n"].state,
-                           cache["m"].state, batch.seg_row0, batch.seg_slot, heads=self.H, key_dim=self.D,
-                           value_dim=self.Dv)
-        y = ops.mlstm_output(o, g, self.norm, self.eps, self.rt.act_dtype, heads=self.H, value_dim=self.Dv)
+        gates = self.gates(x, out_dtype=torch.float32)[:, :2 * self.H]
+        num, nq, coefs = ops.mlstm_scan(q, k, v, gates, self.i_bias, self.f_bias, self.cap, cache["S"].state,
+                                        cache["n"].state, cache["m"].state, batch.seg_row0, batch.seg_slot,
+                                        heads=self.H, key_dim=self.D, value_dim=self.Dv)
+        y = ops.mlstm_output(num, nq, coefs, g, self.norm, self.eps, self.rt.act_dtype, heads=self.H, value_dim=self.Dv)
         return self.o(y, out_dtype=torch.float32, partials_ok=True)   # it goes into the 32-bit residual unrounded

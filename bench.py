@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
     python bench.py --workload qwen3-8b-mixed | qwen3-32b-decode     (two further workloads)
     python bench.py --generate                                       (the decode workload through LLM.generate)
+    python bench.py --workload gufasun [--shape 4b|8b] [--layers L]  (the Gufasun design beside Qwen3 at equal sizes)
 
 A step is one decode step of `batch` requests, each holding a `prompt`-token random prompt
 (prefilled by the engine itself before the clock starts) and growing by one token per step.
@@ -703,6 +704,171 @@ def sweep(args) -> int:
     return 0
 
 
+# ---- the Gufasun design beside Qwen3 at equal sizes -------------------------------------------------------
+# Shapes that resemble a real model's layers: the widths, head counts and feed-forward size of Qwen3-4B / 8B, layers
+# alternating between the matrix memory and the windowed attention, the last attention layer reading the pages of the
+# one before it.  Random weights; the vocabulary is Qwen3's.
+GUFASUN_SHAPES = {"4b": (QWEN3_4B, 20, 1024), "8b": (QWEN3_8B, 32, 2048)}      # (widths, mLSTM heads, window)
+
+
+def gufasun_config(shape: str, layers: int) -> dict:
+    q, mheads, window = GUFASUN_SHAPES[shape]
+    attn = {"heads": q["num_attention_heads"], "kv_heads": q["num_key_value_heads"], "dim": q["head_dim"],
+            "vdim": q["head_dim"], "scale": q["head_dim"] ** -0.5, "softcap": 50.0, "conv": 4, "mask": {"size": window},
+            "q_temp": {"coef": 0.3, "every": 64}}
+    mem = {"heads": mheads, "dim": q["head_dim"], "vdim": q["head_dim"], "gate_cap": 12.0}
+    mlp = {"kind": "dense", "ff": q["intermediate_size"]}
+    out, owner = [], None
+    for i in range(layers):
+        if i % 2 == 0:
+            out.append({"type": "mlstm", "mixer": dict(mem), "mlp": dict(mlp)})
+        else:
+            mixer = dict(attn)
+            if owner is not None and i >= layers - 2:
+                mixer["kv_from"] = owner
+            else:
+                owner = i
+            out.append({"type": "attention", "mixer": mixer, "mlp": dict(mlp)})
+    return {"architecture": "Gufasun", "vocab": q["vocab_size"], "width": q["hidden_size"], "norm": {"eps": 1e-5},
+            "embedding": {"scale": q["hidden_size"] ** 0.5}, "canon": {"taps": 4}, "layers": out}
+
+
+def _kernel_family(name: str) -> str:
+    base = name.split("<")[0].split("(")[0].replace("void ", "").replace("arle::", "").strip()
+    if base.startswith("Cijk") or "gemm" in base.lower() or base.startswith("Custom_Cijk"):
+        return "matrix products (library and own)"
+    return base
+
+
+def gufasun_work(raw: dict, q: dict, tokens: int, batch: int, context: int) -> dict:
+    """Ideal work of the kernels that are new with this design, per step: kernel family -> (bytes, flops) for a step of
+    `tokens` rows, of which `batch` requests (decode: tokens == batch, each with `context` tokens behind it)."""
+    W = raw["width"]
+    a = next(l["mixer"] for l in raw["layers"] if l["type"] == "attention")
+    m = next(l["mixer"] for l in raw["layers"] if l["type"] == "mlstm")
+    n_att = sum(l["type"] == "attention" for l in raw["layers"])
+    n_own = sum(l["type"] == "attention" and "kv_from" not in l["mixer"] for l in raw["layers"])
+    n_mem = len(raw["layers"]) - n_att
+    L = len(raw["layers"])
+    F = raw["layers"][0]["mlp"]["ff"]
+    Q, KV = a["heads"] * a["dim"], a["kv_heads"] * a["dim"]
+    decode = tokens == batch
+    keys = min(a["mask"]["size"], context) if decode else min(a["mask"]["size"], tokens / 2)
+    S = m["heads"] * m["dim"] * m["vdim"]
+    return {
+        "add_layernorm_kernel": ((L + 1) * tokens * W * (4 + 4 + 4 + 4 + 2 + 2), 0),
+        "causal_conv_kernel": (tokens * 2 * 2 * (L * W + n_own * (Q + 2 * KV) + (n_att - n_own) * Q), 0),
+        "polynorm_kernel": (L * tokens * F * 4, 0),
+        "qkv_norm_store_kernel": (tokens * 2 * 2 * (n_own * (Q + 2 * KV) + (n_att - n_own) * Q), 0),
+        "attn_softcap_mfma_kernel": (n_att * batch * 2 * KV * 2 * keys if decode else 0,
+                                     n_att * tokens * keys * a["heads"] * 2 * (a["dim"] + a["vdim"])),
+        "mlstm_memory_kernel": (n_mem * batch * S * 4 * 2, n_mem * tokens * S * 4),
+        "mlstm_gates_kernel": (n_mem * tokens * m["heads"] * m["dim"] * 2 * 2, 0),
+        "mlstm_output_kernel": (n_mem * tokens * m["heads"] * m["vdim"] * (4 + 2 + 2), 0),
+    }
+
+
+def qwen3_work(q: dict, layers: int, tokens: int, batch: int, context: int) -> dict:
+    """The like kernels of the Qwen3 model of the same widths."""
+    W, F = q["hidden_size"], q["intermediate_size"]
+    Q, KV, D = q["num_attention_heads"] * q["head_dim"], q["num_key_value_heads"] * q["head_dim"], q["head_dim"]
+    decode = tokens == batch
+    keys = context if decode else tokens / 2
+    attn = (layers * batch * 2 * KV * 2 * keys if decode else 0, layers * tokens * keys * q["num_attention_heads"] * 4 * D)
+    return {"rmsnorm_vec_kernel": ((2 * layers + 1) * tokens * W * (4 + 4 + 4 + 2), 0),
+            "silu_mul_bf16x8_kernel": (layers * tokens * F * 6, 0),
+            "qk_prep": (layers * tokens * (Q + 2 * KV) * 4, 0),
+            "attn_mfma_kernel": attn, "attn_prefill_dma_kernel": attn, "attn_prefill_lds_kernel": attn}
+
+
+def gufasun_bench(args) -> int:
+    """Prefill and decode throughput of the Gufasun design and of Qwen3 at the same widths and depth, one JSON line
+    each, and the time of a step by kernel family with what each new kernel reaches of its roofline."""
+    import torch
+
+    from arle_amd.config import GufasunConfig, Qwen3Config
+    from arle_amd.engine import Engine, StepEntry
+    from arle_amd.kernels import ops
+
+    layers = args.layers if args.layers != FULL_LAYERS else 8
+    q = dict(GUFASUN_SHAPES[args.shape][0], num_hidden_layers=layers)
+    raw = gufasun_config(args.shape, layers)
+    batch, prompt = args.batch or 8, args.prompt_len
+    models = {"gufasun": ("Gufasun", GufasunConfig.from_dict(raw)), "qwen3": ("Qwen3ForCausalLM", Qwen3Config.from_dict(q))}
+    gen = torch.Generator().manual_seed(1234)
+    toks = lambda n: torch.randint(0, q["vocab_size"], (n,), generator=gen).tolist()
+    lines = []
+    for name, (arch, config) in models.items():
+        engine = Engine.from_config(arch, config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
+                                    max_tokens=(batch + 1) * (prompt + 256), max_slots=batch + 1,
+                                    max_request_tokens=prompt + 256)
+
+        def prefill_once(key):
+            engine.add_request(key)
+            t = toks(prompt)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ops.argmax_rows(engine.step([StepEntry(key, t, [prompt - 1])]))
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            engine.end_request(key)
+            return dt
+
+        for i in range(3):
+            prefill_once(("warm", i))
+        prefill_s = min(prefill_once(("p", i)) for i in range(5))
+        keys = [("d", i) for i in range(batch)]
+        last = []
+        for k in keys:
+            engine.add_request(k)
+            last += ops.argmax_rows(engine.step([StepEntry(k, toks(prompt), [prompt - 1])])).tolist()
+
+        def decode_step():
+            nonlocal last
+            last = ops.argmax_rows(engine.step([StepEntry(k, [t], [0]) for k, t in zip(keys, last)])).tolist()
+
+        for _ in range(args.warmup):
+            decode_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            decode_step()
+        torch.cuda.synchronize()
+        decode_s = (time.perf_counter() - t0) / args.steps
+        line = {"metric": f"{name} at the Qwen3-{args.shape.upper()} widths, {layers} layers, random weights", "dtype": "bf16",
+                "prefill_tok_s": round(prompt / prefill_s, 1), "prefill_ms": round(prefill_s * 1e3, 3), "prompt": prompt,
+                "decode_tok_s": round(batch / decode_s, 1), "decode_ms": round(decode_s * 1e3, 3), "batch": batch}
+        if not args.no_parts:
+            engine.use_graphs = False        # the profiler names the kernels of eager steps
+            engine.add_request("prof")
+            t = toks(prompt)
+            pre, dec = profiled_steps(torch, [lambda: engine.step([StepEntry("prof", t, [prompt - 1])]), decode_step])
+            engine.end_request("prof")
+            work = {"prefill": gufasun_work(raw, q, prompt, 1, 0) if name == "gufasun" else qwen3_work(q, layers, prompt, 1, 0),
+                    "decode": gufasun_work(raw, q, batch, batch, prompt) if name == "gufasun" else qwen3_work(q, layers, batch, batch, prompt)}
+            for phase, step in (("prefill", pre), ("decode", dec)):
+                fam: dict = {}
+                for kname, us in step:
+                    f = fam.setdefault(_kernel_family(kname), [0, 0.0])
+                    f[0] += 1
+                    f[1] += us
+                table = {}
+                for f, (count, us) in sorted(fam.items(), key=lambda kv: -kv[1][1]):
+                    row = {"launches": count, "us": round(us, 1)}
+                    match = next((w for key, w in work[phase].items() if f.startswith(key)), None)
+                    if match is not None and us > 0:
+                        row["of_roofline"] = round(max(match[0] / (PEAK_HBM_GBS * 1e9), match[1] / PEAK_FLOPS["bf16"]) / (us * 1e-6), 4)
+                    table[f] = row
+                line[phase + "_kernels"] = table
+        print(json.dumps(line), flush=True)
+        lines.append(line)
+        for k in keys:
+            engine.end_request(k)
+        del engine
+        torch.cuda.empty_cache()
+    return 0
+
+
 def main() -> int:
     global PAGE, PROMPT
     ap = argparse.ArgumentParser()
@@ -745,8 +911,10 @@ def main() -> int:
                          "and write the table that ARLE_AMD_PRODUCT_TABLE / ops.load_product_table reads; WIDTHS: 4b, 8b, "
                          "32b or hidden,q_width,kv_width,intermediate[,vocabulary]")
     ap.add_argument("--out", default=None, help="--tune-products: the table's file (default: product_table_<widths>.json)")
-    ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode"],
-                    help="qwen3-4b is the default run; the other two are further workloads at larger shapes")
+    ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode", "gufasun"],
+                    help="qwen3-4b is the default run; the next two are further workloads at larger shapes; gufasun: "
+                         "the Gufasun design beside Qwen3 at equal widths and depth (--shape, --layers, --batch, --prompt-len)")
+    ap.add_argument("--shape", default="4b", choices=["4b", "8b"], help="--workload gufasun: whose widths")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
@@ -766,6 +934,8 @@ def main() -> int:
         return generate_workload(args)
     if args.gaps:
         return step_gaps(args)
+    if args.workload == "gufasun":
+        return gufasun_bench(args)
     if args.workload == "qwen3-4b" and args.batch is None:
         args.batch = 8
     if args.workload != "qwen3-4b":
