@@ -18,66 +18,54 @@ namespace arle {
 
 constexpr int kCapMaxD = 512;
 
+// One wave a (row, head of q, k or v).  T: the element type of q, k, v and the pages; the loads of a head are typed and
+// unconditional (an element past the head's size reads the head's last one and is dropped).
+template <typename T>
 __global__ __launch_bounds__(kWave) void qkv_norm_store_kernel(
-    void* __restrict__ q, long long q_stride, const void* __restrict__ k, long long k_stride,
-    const void* __restrict__ v, long long v_stride, int dtype, const void* __restrict__ q_weight,
-    const void* __restrict__ k_weight, int w_dtype, float eps, float temp_coef, int temp_every,
-    const int* __restrict__ positions, const int* __restrict__ slot_of_token, const int* __restrict__ block_table,
-    int table_stride, void* __restrict__ k_pages, void* __restrict__ v_pages, int nq, int nkv, int Dk, int Dv,
-    int page_size) {
+    T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride, const T* __restrict__ v,
+    long long v_stride, const void* __restrict__ q_weight, const void* __restrict__ k_weight, int w_dtype, float eps,
+    float temp_coef, int temp_every, const int* __restrict__ positions, const int* __restrict__ slot_of_token,
+    const int* __restrict__ block_table, int table_stride, T* __restrict__ k_pages, T* __restrict__ v_pages, int nq,
+    int nkv, int Dk, int Dv, int page_size) {
   const int64_t t = blockIdx.x;
   const int y = blockIdx.y, lane = threadIdx.x;
   const int pos = positions[t];
-  if (y < nq) {
-    float x[kCapMaxD / kWave];
+  if (y < nq + nkv) {
+    const bool is_q = y < nq;
+    const int g = is_q ? y : y - nq;
+    const T* src = is_q ? q + t * q_stride + g * Dk : k + t * k_stride + g * Dk;
+    const void* weight = is_q ? q_weight : k_weight;
+    float x[kCapMaxD / kWave], w[kCapMaxD / kWave];
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < kCapMaxD / kWave; ++j) {
       const int d = lane + j * kWave;
-      x[j] = d < Dk ? load_as_float(q, dtype, t * q_stride + y * Dk + d) : 0.f;
-      ss = fmaf(x[j], x[j], ss);
+      if (j * kWave < Dk) {
+        x[j] = to_float(src[min(d, Dk - 1)]);
+        w[j] = weight ? load_as_float(weight, w_dtype, min(d, Dk - 1)) : 1.0f;
+        if (d < Dk) ss = fmaf(x[j], x[j], ss);
+      }
     }
     float f = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(Dk) + eps);
-    const float temp = temp_coef != 0.f ? 1.0f + temp_coef * logf(static_cast<float>((pos + 1) / temp_every + 1)) : 1.0f;
+    T* dst;
+    if (is_q) {
+      if (temp_coef != 0.f) f *= 1.0f + temp_coef * logf(static_cast<float>((pos + 1) / temp_every + 1));
+      dst = q + t * q_stride + g * Dk;
+    } else {
+      const int page = block_table[static_cast<int64_t>(slot_of_token[t]) * table_stride + pos / page_size];
+      dst = k_pages + ((static_cast<int64_t>(page) * nkv + g) * page_size + pos % page_size) * Dk;
+    }
 #pragma unroll
     for (int j = 0; j < kCapMaxD / kWave; ++j) {
       const int d = lane + j * kWave;
-      if (d < Dk) {
-        const float w = q_weight ? load_as_float(q_weight, w_dtype, d) : 1.0f;
-        store_from_float(q, dtype, t * q_stride + y * Dk + d, x[j] * f * w * temp);
-      }
+      if (j * kWave < Dk && d < Dk) dst[d] = from_float<T>(x[j] * f * w[j]);
     }
     return;
   }
   const int page = block_table[static_cast<int64_t>(slot_of_token[t]) * table_stride + pos / page_size];
-  const int in_page = pos % page_size;
-  if (y < nq + nkv) {
-    const int g = y - nq;
-    float x[kCapMaxD / kWave];
-    float ss = 0.f;
-#pragma unroll
-    for (int j = 0; j < kCapMaxD / kWave; ++j) {
-      const int d = lane + j * kWave;
-      x[j] = d < Dk ? load_as_float(k, dtype, t * k_stride + g * Dk + d) : 0.f;
-      ss = fmaf(x[j], x[j], ss);
-    }
-    const float f = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(Dk) + eps);
-    const int64_t base = ((static_cast<int64_t>(page) * nkv + g) * page_size + in_page) * Dk;
-#pragma unroll
-    for (int j = 0; j < kCapMaxD / kWave; ++j) {
-      const int d = lane + j * kWave;
-      if (d < Dk) {
-        const float w = k_weight ? load_as_float(k_weight, w_dtype, d) : 1.0f;
-        store_from_float(k_pages, dtype, base + d, x[j] * f * w);
-      }
-    }
-    return;
-  }
   const int g = y - nq - nkv;
-  const int64_t base = (static_cast<int64_t>(page) * nkv + g) * Dv * page_size + in_page;
-  for (int d = lane; d < Dv; d += kWave)
-    store_from_float(v_pages, dtype, base + static_cast<int64_t>(d) * page_size,
-                     load_as_float(v, dtype, t * v_stride + g * Dv + d));
+  T* dst = v_pages + (static_cast<int64_t>(page) * nkv + g) * Dv * page_size + pos % page_size;
+  for (int d = lane; d < Dv; d += kWave) dst[static_cast<int64_t>(d) * page_size] = v[t * v_stride + g * Dv + d];
 }
 
 template <typename T>
@@ -171,9 +159,19 @@ extern "C" int arle_qkv_norm_store(void* q, long long q_stride, const void* k, l
   if (tokens == 0) return 0;
   if (Dk > kCapMaxD || Dk < 1 || nq + 2 * nkv > 65535 || (temp_coef != 0.f && temp_every < 1))
     return static_cast<int>(hipErrorInvalidValue);
-  qkv_norm_store_kernel<<<dim3(tokens, nq + 2 * nkv), kWave, 0, static_cast<hipStream_t>(stream)>>>(
-      q, q_stride, k, k_stride, v, v_stride, dtype, q_weight, k_weight, w_dtype, eps, temp_coef, temp_every, positions,
-      slot_of_token, block_table, table_stride, k_pages, v_pages, nq, nkv, Dk, Dv, page_size);
+  const dim3 grid(tokens, nq + 2 * nkv);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == kF32) {
+    qkv_norm_store_kernel<float><<<grid, kWave, 0, s>>>(
+        static_cast<float*>(q), q_stride, static_cast<const float*>(k), k_stride, static_cast<const float*>(v), v_stride,
+        q_weight, k_weight, w_dtype, eps, temp_coef, temp_every, positions, slot_of_token, block_table, table_stride,
+        static_cast<float*>(k_pages), static_cast<float*>(v_pages), nq, nkv, Dk, Dv, page_size);
+  } else {
+    qkv_norm_store_kernel<bf16><<<grid, kWave, 0, s>>>(
+        static_cast<bf16*>(q), q_stride, static_cast<const bf16*>(k), k_stride, static_cast<const bf16*>(v), v_stride,
+        q_weight, k_weight, w_dtype, eps, temp_coef, temp_every, positions, slot_of_token, block_table, table_stride,
+        static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), nq, nkv, Dk, Dv, page_size);
+  }
   return launch_status();
 }
 

@@ -756,9 +756,9 @@ def gufasun_work(raw: dict, q: dict, tokens: int, batch: int, context: int) -> d
     keys = min(a["mask"]["size"], context) if decode else min(a["mask"]["size"], tokens / 2)
     S = m["heads"] * m["dim"] * m["vdim"]
     return {
-        "add_layernorm_kernel": ((L + 1) * tokens * W * (4 + 4 + 4 + 4 + 2 + 2), 0),
-        "causal_conv_kernel": (tokens * 2 * 2 * (L * W + n_own * (Q + 2 * KV) + (n_att - n_own) * Q), 0),
-        "polynorm_kernel": (L * tokens * F * 4, 0),
+        "add_layernorm": ((L + 1) * tokens * W * (4 + 4 + 4 + 4 + 2 + 2), 0),
+        "causal_conv": (tokens * 2 * 2 * (L * W + n_own * (Q + 2 * KV) + (n_att - n_own) * Q), 0),
+        "polynorm": (L * tokens * F * 4, 0),
         "qkv_norm_store_kernel": (tokens * 2 * 2 * (n_own * (Q + 2 * KV) + (n_att - n_own) * Q), 0),
         "attn_softcap_mfma_kernel": (n_att * batch * 2 * KV * 2 * keys if decode else 0,
                                      n_att * tokens * keys * a["heads"] * 2 * (a["dim"] + a["vdim"])),
@@ -775,7 +775,8 @@ def qwen3_work(q: dict, layers: int, tokens: int, batch: int, context: int) -> d
     decode = tokens == batch
     keys = context if decode else tokens / 2
     attn = (layers * batch * 2 * KV * 2 * keys if decode else 0, layers * tokens * keys * q["num_attention_heads"] * 4 * D)
-    return {"rmsnorm_vec_kernel": ((2 * layers + 1) * tokens * W * (4 + 4 + 4 + 2), 0),
+    return {"rmsnorm_vec_kernel": ((layers + 1) * tokens * W * (4 + 4 + 4 + 2), 0),
+            "add_stack_rmsnorm_kernel": (layers * tokens * W * (4 + 4 + 4 + 2), 0),
             "silu_mul_bf16x8_kernel": (layers * tokens * F * 6, 0),
             "qk_prep": (layers * tokens * (Q + 2 * KV) * 4, 0),
             "attn_mfma_kernel": attn, "attn_prefill_dma_kernel": attn, "attn_prefill_lds_kernel": attn}

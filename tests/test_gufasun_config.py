@@ -87,3 +87,28 @@ def test_a_single_need_still_stands_alone():
     cache = CacheManager([StateNeed((3,), torch.float32), PagedNeed(2, 8), None], page_size=4, num_pages=4, max_slots=2,
                          max_request_tokens=16, readers={2: 1})
     assert isinstance(cache.view(0), StateView) and cache.view(1).writes and not cache.view(2).writes
+
+
+def test_the_command_line_writes_a_random_model_folder_of_this_design(tmp_path, capsys):
+    import json
+    import os
+
+    from safetensors.torch import load_file
+
+    from arle_amd.cli import main
+
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(TINY_Q))
+    out = str(tmp_path / "model")
+    assert main(["random-weights", "--config", str(config), "--out", out, "--seed-weights", "3"]) == 0
+    assert capsys.readouterr().out.strip() == out
+    assert json.load(open(os.path.join(out, "config.json")))["architecture"] == "Gufasun"
+    names = set(load_file(os.path.join(out, "model.safetensors")))
+    assert {"embed", "head", "final.norm", "l0.mix.i.b", "l1.mix.r2", "l2.mix.k.conv", "l2.canon1"} <= names
+    assert "l1.mix.q.conv" not in names       # that layer has no convolution on q, k and v
+    # a folder of this design that is damaged ends like any other: one line, exit code 1
+    bad = dict(TINY_Q, layers=[dict(TINY_Q["layers"][0], type="gru")])
+    (tmp_path / "bad").mkdir()
+    (tmp_path / "bad" / "config.json").write_text(json.dumps(bad))
+    assert main(["--model-path", str(tmp_path / "bad"), "run", "--prompt-ids", "1,2"]) == 1
+    assert "unknown layer type" in capsys.readouterr().err
