@@ -714,9 +714,9 @@ GUFASUN_SHAPES = {"4b": (QWEN3_4B, 20, 1024), "8b": (QWEN3_8B, 32, 2048)}      #
 def gufasun_config(shape: str, layers: int) -> dict:
     q, mheads, window = GUFASUN_SHAPES[shape]
     attn = {"heads": q["num_attention_heads"], "kv_heads": q["num_key_value_heads"], "dim": q["head_dim"],
-            "vdim": q["head_dim"], "scale": q["head_dim"] ** -0.5, "softcap": 50.0, "conv": 4, "mask": {"size": window},
-            "q_temp": {"coef": 0.3, "every": 64}}
-    mem = {"heads": mheads, "dim": q["head_dim"], "vdim": q["head_dim"], "gate_cap": 12.0}
+            "vdim": q["head_dim"], "scale": q["head_dim"] ** -0.5, "softcap": 30.0, "conv": 4, "mask": {"size": window},
+            "q_temp": {"coef": 0.25, "every": 128}}
+    mem = {"heads": mheads, "dim": q["head_dim"], "vdim": q["head_dim"], "gate_cap": 15.0}
     mlp = {"kind": "dense", "ff": q["intermediate_size"]}
     out, owner = [], None
     for i in range(layers):
@@ -729,8 +729,8 @@ def gufasun_config(shape: str, layers: int) -> dict:
             else:
                 owner = i
             out.append({"type": "attention", "mixer": mixer, "mlp": dict(mlp)})
-    return {"architecture": "Gufasun", "vocab": q["vocab_size"], "width": q["hidden_size"], "norm": {"eps": 1e-5},
-            "embedding": {"scale": q["hidden_size"] ** 0.5}, "canon": {"taps": 4}, "layers": out}
+    return {"architecture": "Gufasun", "vocab": q["vocab_size"], "width": q["hidden_size"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": 32.0}, "canon": {"taps": 4}, "layers": out}
 
 
 def _kernel_family(name: str) -> str:
