@@ -41,8 +41,7 @@ class AttentionMixer:
                 "softcap": self.softcap, "conv": self.conv}
         if self.window is not None:
             body["mask"] = {"size": self.window}
-        if self.temp_coef:
-            body["q_temp"] = {"coef": self.temp_coef, "every": self.temp_every}
+        body["q_temp"] = {"coef": self.temp_coef, "every": self.temp_every}
         if self.kv_from is not None:
             body["kv_from"] = self.kv_from
         return body

@@ -64,16 +64,18 @@ def attention_mixer(h, p, m, eps, keys, values):
         q = causal_conv(q, p["q.conv"])
     q = rms_unit(q.view(T, H, D), eps) * p["q.norm"]
     pos = torch.arange(T, dtype=h.dtype)
-    temp = 1 + m["q_temp"]["coef"] * torch.log(torch.floor((pos + 1) / m["q_temp"]["every"]) + 1)
-    q = q * temp[:, None, None]
-    cap, window = m["softcap"], m["mask"]["size"]
+    if m.get("q_temp"):
+        temp = 1 + m["q_temp"]["coef"] * torch.log(torch.floor((pos + 1) / m["q_temp"]["every"]) + 1)
+        q = q * temp[:, None, None]
+    cap, window = m.get("softcap", 0.0), m["mask"]["size"]
     out = torch.zeros(T, H, values.shape[-1], dtype=h.dtype)
     for hq in range(H):
         g = hq // (H // G)
         for i in range(T):
             lo = max(0, i - window + 1)
             s = (keys[lo:i + 1, g] @ q[i, hq]) * m["scale"]
-            s = cap * torch.tanh(s / cap)
+            if cap:
+                s = cap * torch.tanh(s / cap)
             dist = (i - torch.arange(lo, i + 1)).to(h.dtype)
             s = s - p["r1"][hq] * torch.log1p(p["r2"][hq] * dist)
             out[i, hq] = torch.softmax(s, 0) @ values[lo:i + 1, g]

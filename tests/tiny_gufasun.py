@@ -6,6 +6,8 @@ Q: the values that often coincide are made to differ, and the ones that are ofte
 convolution, one kv head a q head, a window of one page and one of a single key, a temperature period of 1, one
 mLSTM head, no convolution on q, k and v in one layer, a value size that is no multiple of 16.
 R: wider heads (a key size over 64, a value size over 64 that is no multiple of 64) and windows of several pages.
+S: nothing but matrix memories (no paged cache at all).  T: nothing but attention, five q heads a kv head, a key size
+that is a multiple of 8 only, a reader right behind its owner, and no feed-forward anywhere.
 """
 from __future__ import annotations
 
@@ -54,8 +56,18 @@ TINY_R = {"architecture": ARCH, "vocab": 300, "width": 96, "norm": {"eps": 1e-5}
                      layer("mlstm", mlstm(2, 80, 96), 160),
                      layer("attention", attention(4, 2, 80, 96, window=33, conv=2, scale=0.2, kv_from=0), 128)]}
 
+TINY_S = {"architecture": ARCH, "vocab": 120, "width": 48, "norm": {"eps": 1e-5}, "embedding": {"scale": 2.0},
+          "canon": {"taps": 2},
+          "layers": [layer("mlstm", mlstm(2, 20, 36), 64), layer("mlstm", mlstm(4, 8, 12, cap=5.0), None)]}
+
+TINY_T = {"architecture": ARCH, "vocab": 150, "width": 60, "norm": {"eps": 1e-5}, "embedding": {"scale": 3.0},
+          "canon": {"taps": 5},
+          "layers": [layer("attention", attention(5, 1, 24, 48, window=19, conv=3), None),
+                     layer("attention", attention(5, 1, 24, 48, window=50, conv=4, softcap=0.0, coef=0.0, kv_from=0), None)]}
+
 # name -> (config, page size, weight std, norm std, seed)
-TINY = {"P": (TINY_P, 4, 0.15, 0.1, 5), "Q": (TINY_Q, 8, 0.2, 0.2, 6), "R": (TINY_R, 16, 0.1, 0.1, 7)}
+TINY = {"P": (TINY_P, 4, 0.15, 0.1, 5), "Q": (TINY_Q, 8, 0.2, 0.2, 6), "R": (TINY_R, 16, 0.1, 0.1, 7),
+        "S": (TINY_S, 16, 0.2, 0.1, 8), "T": (TINY_T, 16, 0.2, 0.1, 9)}
 
 
 def make_model_dir(tmp_path, name: str) -> str:
