@@ -11,7 +11,7 @@ Per token, with h the mixer's input, H heads, key size D, value size Dv:
 
 S, n and m start at zero and live in 32-bit state slots `[H, D, Dv]`, `[H, D]`, `[H]` of the request; the gates'
 projections, the gates, the recurrence and the head norm are 32-bit in every mode.  q, k, v and the output gate
-come from one fused product; the two gate projections are a float32 product of their own.
+come from one fused product that hands over its 32-bit sums; the two gate projections are a product of their own.
 """
 from __future__ import annotations
 
@@ -80,7 +80,9 @@ class MLSTMMixer(Part):
     def forward(self, x, batch, cache):
         """x [T, W] -> [T, W], or a float32 stack [S, T, W] to be added in order (see Linear)."""
         qk, vw = self.H * self.D, self.H * self.Dv
-        p = self.qkvg(x)
+        # 32-bit sums out of the product: q and k meet in dot products whose terms cancel (a request's first rows hang
+        # on a single one), and what rounding them to bfloat16 costs there is ten times a usual row's error
+        p = self.qkvg(x, out_dtype=torch.float32)
         q, k, v, g = p[:, :qk], p[:, qk:2 * qk], p[:, 2 * qk:2 * qk + vw], p[:, 2 * qk + vw:]
         gates = self.gates(x, out_dtype=torch.float32)[:, :2 * self.H]
         num, nq, coefs = ops.mlstm_scan(q, k, v, gates, self.i_bias, self.f_bias, self.cap, cache["S"].state,
