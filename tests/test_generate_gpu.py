@@ -33,7 +33,7 @@ def _plain_greedy(cfg, weights, prompt, n):
 
 
 def test_greedy_generation_equals_the_plain_implementation(folders):
-    # configuration A of the task: prompts of 5 / 11 / 17 tokens, 8 greedy tokens each
+    # configuration A: prompts of 5 / 11 / 17 tokens, 8 greedy tokens each
     cfg, weights = read_folder(folders["A"])
     prompts = [random_tokens(n, cfg["vocab_size"], 70 + n) for n in (5, 11, 17)]
     want = [_plain_greedy(cfg, weights, p, 8) for p in prompts]
@@ -58,7 +58,7 @@ def test_bfloat16_greedy_picks_near_best_tokens(folders):
 
 
 def test_temperature_sampling_with_portions_equals_plain_inverse_cdf(folders):
-    # configuration B of the task: prompts of 1 / 9 / 23 / 40, portions of 16, temperature 0.8, 6 tokens
+    # configuration B: prompts of 1 / 9 / 23 / 40, portions of 16, temperature 0.8, 6 tokens
     cfg, weights = read_folder(folders["B"])
     prompts = [random_tokens(n, cfg["vocab_size"], 90 + n) for n in (1, 9, 23, 40)]
     llm = LLM(folders["B"], dtype="float32", page_size=TINY["B"][1], kv_cache_tokens=512, max_seq_len=128,
