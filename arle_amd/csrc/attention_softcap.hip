@@ -223,6 +223,10 @@ __device__ __forceinline__ float fast_tanh(float x) {
   return fmaf(-2.0f, __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * x)), 1.0f);
 }
 
+// Portions do not fetch a tile ahead: with thousands of waves, more of them a SIMD hide the loads better than a second
+// set of registers (2,048 rows behind a window of 1,024: 213 us a layer without, 288 with).
+constexpr bool kCapRowsAhead = false;
+
 struct CapArgs {
   const bf16* q; long long q_stride;
   bf16* out; long long o_stride;
@@ -233,6 +237,7 @@ struct CapArgs {
   float scale, cap;
   const void* r1; const void* r2; int r_dtype;
   int window;
+  int merge_floats;   // floats of dynamic LDS in front of the page ids
 };
 
 // KC: chunks of 32 of the key size held (Dk <= 32 KC); VC: chunks of 16 of the value size (Dv <= 16 VC).
@@ -241,7 +246,7 @@ struct CapArgs {
 // and the waves of a workgroup are WAVES q heads of one kv head on the same rows, so that they fetch the same tiles.
 template <int KC, int VC, bool HEADS, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const CapArgs a) {
-  extern __shared__ float merge_lds[];   // HEADS: [WAVES][n_vc][64 lanes][4], then m [WAVES][16], l [WAVES][16]
+  extern __shared__ float merge_lds[];   // HEADS: [WAVES][n_vc][64 lanes][4], then m [WAVES][16], l [WAVES][16]; then page ids
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n = lane % 16, g = lane / 16;
   const int group = a.nq / a.nkv;
   int seg, row, head, kvh, first_row, last_row;
@@ -291,9 +296,8 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
   const bf16* qr = a.q + static_cast<int64_t>(row) * a.q_stride + head * a.Dk;
 #pragma unroll
   for (int c = 0; c < KC; ++c) {
-    u32x4_t raw = {0, 0, 0, 0};
-    if (c < n_kc && 32 * c + 8 * g < a.Dk) raw = *reinterpret_cast<const u32x4_t*>(qr + 32 * c + 8 * g);
-    qreg[c] = __builtin_bit_cast(bf16x8_t, raw);
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(qr + min(32 * c + 8 * g, a.Dk - 8));
+    qreg[c] = __builtin_bit_cast(bf16x8_t, 32 * c + 8 * g < a.Dk ? raw : u32x4_t{0, 0, 0, 0});
   }
   f32x4_t acc[VC];
 #pragma unroll
@@ -308,35 +312,35 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
 
   // Every load of a tile (K rows, V columns, after the two page ids) is sent a tile ahead, while the tile before it
   // is worked through; a tile past the last is the last one again, fetched and dropped.
-  // The ids of the first 128 pages that the item sees are fetched once, a page a lane and two a lane, and read from
-  // there (a scalar lane read): a tile's loads then wait for no load of a page id before them.
-  const int page_first = key_lo / a.page_size;
-  const int held0 = table[min(page_first + lane, last_entry)], held1 = table[min(page_first + kWave + lane, last_entry)];
+  // The ids of the pages that the item sees are put into LDS once: a tile's loads then follow no load of a page id,
+  // and the reads of LDS are counted apart from the loads from memory, so they disturb no wait for those.
+  const int page_first = (key_lo / 32 * 32) / a.page_size;   // the page of the first tile's first key, which may lie in front of key_lo's
+  int* page_lds = reinterpret_cast<int*>(merge_lds) + a.merge_floats;
+  for (int i = threadIdx.x; i <= (tile_last * 32 + 31) / a.page_size - page_first; i += WAVES * kWave)
+    page_lds[i] = table[min(page_first + i, last_entry)];
+  __syncthreads();
   auto load_tile = [&](int tile, u32x4_t (&kraw)[2][KC], u32x4_t (&vraw)[VC]) {
     const int key0 = min(tile, tile_last) * 32;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int kb = key0 + 16 * half;
-      const int rel = kb / a.page_size - page_first;
-      const int entry = rel < kWave         ? __builtin_amdgcn_readlane(held0, rel)
-                        : rel < 2 * kWave ? __builtin_amdgcn_readlane(held1, rel - kWave)
-                                          : table[min(kb / a.page_size, last_entry)];
-      const int64_t page = max(entry, 0);
+      const int64_t page = max(page_lds[max(kb / a.page_size - page_first, 0)], 0);
       const int in_page = kb % a.page_size;
       const bf16* kr = a.k_pages + page * k_page + k_head + static_cast<int64_t>(in_page + n) * a.Dk;
+      // no load stands under a condition (one would make every later wait a wait for all loads in flight): a piece
+      // past the head's size is the head's last piece again, zeroed or left unused afterwards
 #pragma unroll
       for (int c = 0; c < KC; ++c) {
-        kraw[half][c] = u32x4_t{0, 0, 0, 0};
-        if (c < n_kc && 32 * c + 8 * g < a.Dk) kraw[half][c] = *reinterpret_cast<const u32x4_t*>(kr + 32 * c + 8 * g);
+        const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(kr + min(32 * c + 8 * g, a.Dk - 8));
+        kraw[half][c] = 32 * c + 8 * g < a.Dk ? raw : u32x4_t{0, 0, 0, 0};
       }
 #pragma unroll
       for (int c = 0; c < VC; ++c) {
-        if (c < n_vc) {
-          const bf16* vr = a.v_pages + page * v_page + v_head + static_cast<int64_t>(16 * c + n) * a.page_size + in_page + 4 * g;
-          const u32x2_t two = *reinterpret_cast<const u32x2_t*>(vr);
-          vraw[c][2 * half] = two[0];
-          vraw[c][2 * half + 1] = two[1];
-        }
+        const bf16* vr = a.v_pages + page * v_page + v_head + static_cast<int64_t>(min(16 * c + n, a.Dv - 1)) * a.page_size +
+                         in_page + 4 * g;
+        const u32x2_t two = *reinterpret_cast<const u32x2_t*>(vr);
+        vraw[c][2 * half] = two[0];
+        vraw[c][2 * half + 1] = two[1];
       }
     }
   };
@@ -404,7 +408,7 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
     }
   };
 
-  if (HEADS) {
+  if (HEADS || kCapRowsAhead) {
     // a decoded row's waves are few and each walks a chain of tiles: the next tile's loads fly while this one is worked
     u32x4_t k_even[2][KC], v_even[VC], k_odd[2][KC], v_odd[VC];
     if (tile_first <= tile_last) load_tile(tile_first, k_even, v_even);
@@ -416,8 +420,6 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
       work_tile(tile + tile_step, k_odd, v_odd);
     }
   } else {
-    // portions bring thousands of waves: more of them a SIMD hide the loads better than a second set of registers
-    // (measured: 2,048 rows behind a window of 1,024, 256 us a layer this way, 388 with the tile fetched ahead)
     u32x4_t k_now[2][KC], v_now[VC];
     for (int tile = tile_first; tile <= tile_last; ++tile) {
       load_tile(tile, k_now, v_now);
@@ -498,11 +500,18 @@ extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* o
   hipStream_t s = static_cast<hipStream_t>(stream);
   const CapArgs a{static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), o_stride,
                   static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages), block_table, table_stride,
-                  seg_row0, seg_slot, seg_start, segments, nq, nkv, Dk, Dv, page_size, scale, cap, r1, r2, r_dtype, window};
+                  seg_row0, seg_slot, seg_start, segments, nq, nkv, Dk, Dv, page_size, scale, cap, r1, r2, r_dtype, window,
+                  heads_mode ? kCapSplitWaves * ((Dv / 16) * kWave * 4 + 32) : 0};
+  // pages an item can see: its rows' windows (or everything the block table maps) and the tiles' rounding to 32 keys;
+  // nothing of a step's lengths, so that a captured launch holds for every later step of its shape
+  const long long mapped = static_cast<long long>(table_stride) * page_size;
+  const long long keys_seen = (window > 0 && window + 16 < mapped ? window + 16 : mapped) + 64;
+  const size_t page_bytes = (static_cast<size_t>(keys_seen) / page_size + 2) * sizeof(int);
+  if (page_bytes > 48 * 1024) return static_cast<int>(hipErrorInvalidValue);
   const int size = (Dk + 1) / 2 > Dv ? (Dk + 1) / 2 : Dv;   // Dk counts half: a chunk of keys is 32 wide, of values 16
   const int group = nq / nkv;
   const int head_waves = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);   // q heads of one kv head that share a workgroup
-  const size_t merge_bytes = static_cast<size_t>(kCapSplitWaves) * ((Dv / 16) * kWave * 4 + 32) * sizeof(float);
+  const size_t merge_bytes = static_cast<size_t>(kCapSplitWaves) * ((Dv / 16) * kWave * 4 + 32) * sizeof(float) + page_bytes;
 #define ARLE_CAP(KC, VC)                                                                                           \
   do {                                                                                                             \
     if (heads_mode) {                                                                                              \
@@ -510,7 +519,7 @@ extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* o
       if (!raised && merge_bytes > 48 * 1024) {                                                                    \
         const hipError_t e = hipFuncSetAttribute(                                                                  \
             reinterpret_cast<const void*>(&attn_softcap_mfma_kernel<KC, VC, true, kCapSplitWaves>),                \
-            hipFuncAttributeMaxDynamicSharedMemorySize, kCapSplitWaves * (VC * kWave * 4 + 32) * 4);              \
+            hipFuncAttributeMaxDynamicSharedMemorySize, kCapSplitWaves * (VC * kWave * 4 + 32) * 4 + 48 * 1024);              \
         if (e != hipSuccess) return static_cast<int>(e);                                                           \
         raised = true;                                                                                             \
       }                                                                                                            \
@@ -518,11 +527,11 @@ extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* o
           <<<dim3(segments, nkv), kCapSplitWaves * kWave, merge_bytes, s>>>(a);                                    \
     }                                                                                                              \
     else if (head_waves == 4)                                                                                      \
-      attn_softcap_mfma_kernel<KC, VC, false, 4><<<dim3(row_blocks, nq / 4), 4 * kWave, 0, s>>>(a);                \
+      attn_softcap_mfma_kernel<KC, VC, false, 4><<<dim3(row_blocks, nq / 4), 4 * kWave, page_bytes, s>>>(a);                \
     else if (head_waves == 2)                                                                                      \
-      attn_softcap_mfma_kernel<KC, VC, false, 2><<<dim3(row_blocks, nq / 2), 2 * kWave, 0, s>>>(a);                \
+      attn_softcap_mfma_kernel<KC, VC, false, 2><<<dim3(row_blocks, nq / 2), 2 * kWave, page_bytes, s>>>(a);                \
     else                                                                                                           \
-      attn_softcap_mfma_kernel<KC, VC, false, 1><<<dim3(row_blocks, nq), kWave, 0, s>>>(a);                        \
+      attn_softcap_mfma_kernel<KC, VC, false, 1><<<dim3(row_blocks, nq), kWave, page_bytes, s>>>(a);                        \
   } while (0)
   if (size <= 64) {
     ARLE_CAP(4, 4);

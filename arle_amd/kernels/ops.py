@@ -1651,6 +1651,14 @@ def attn_softcap_mfma_supported(dtype, key_dim: int, value_dim: int, page_size: 
             and key_dim <= CAP_MFMA_MAX_DIM and value_dim <= CAP_MFMA_MAX_DIM)
 
 
+def attn_softcap_mfma_fits(window: int, table_width: int, page_size: int) -> bool:
+    """Whether the ids of the pages that a row's keys span (its window, or all that the block table maps) fit where
+    the matrix-core kernel keeps them."""
+    mapped = table_width * page_size
+    seen = (window + 16 if 0 < window and window + 16 < mapped else mapped) + 64
+    return (seen // page_size + 2) * 4 <= 48 * 1024
+
+
 def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *, max_qlen: int,
                       num_q_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
                       softcap: float = 0.0, r1=None, r2=None, window: int = 0):
@@ -1678,6 +1686,8 @@ def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot,
     if r1 is not None:
         _need(r1.shape == (num_q_heads,) and r2.shape == (num_q_heads,) and r1.dtype == r2.dtype and r1.dtype in _CODES
               and r1.is_contiguous() and r2.is_contiguous(), "r1, r2 must be [heads] of one type")
+    _need(attn_softcap_mfma_fits(window, block_table.shape[1], page_size),
+          "the keys a row sees span more pages than the kernel holds ids for")
     heads_mode = max_qlen == 1 and group <= 16 and segments == tokens
     row_blocks = tokens // 16 + segments      # no fewer than the sixteen-row blocks of all segments together
     lib.call("arle_attn_softcap_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(),

@@ -156,7 +156,8 @@ def softcap_attention(q, out, kv, batch, *, num_q_heads, num_kv_heads, key_dim, 
     kernel takes run there; float32 pages, and every other shape, run the fixed-order kernel (the true 32-bit path)."""
     common = dict(num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, key_dim=key_dim, value_dim=value_dim,
                   page_size=kv.page_size, scale=scale, softcap=softcap, r1=r1, r2=r2, window=window)
-    if ops.attn_softcap_mfma_supported(q.dtype, key_dim, value_dim, kv.page_size, num_q_heads // num_kv_heads):
+    if (ops.attn_softcap_mfma_supported(q.dtype, key_dim, value_dim, kv.page_size, num_q_heads // num_kv_heads)
+            and ops.attn_softcap_mfma_fits(window, kv.block_table.shape[1], kv.page_size)):
         ops.attn_softcap_mfma(q, out, kv.pages["k"], kv.pages["v"], kv.block_table, batch.seg_row0, batch.seg_slot,
                               batch.seg_start, max_qlen=batch.max_qlen, **common)
     else:
