@@ -4,6 +4,11 @@
 //   s_ij = scale (q_i . k_j);   s <- cap tanh(s / cap)  (cap > 0);   s <- s - r1_h ln(1 + r2_h (i - j))  (r1 given)
 //   o_i  = sum_j softmax_j(s_ij) v_j     over  max(0, i - window + 1) <= j <= i   (window 0: every earlier key)
 //
+// Two further options: `chunk` > 0 lets row i see only the keys of its own chunk, floor(i / chunk) chunk <= j <= i
+// (chunks are counted from position 0 of the request); `sink` [heads] adds exp(sink_h) to the softmax's denominator,
+// a term without key or value.  `wide_norm_store` prepares the operands of an attention whose q and k are RMS-normed
+// over the whole projection (all heads at once) and whose values may be mixed with another layer's.
+//
 // q head h reads kv head h / (nq / nkv).  Keys lie in pages [page, nkv, slot, Dk], values d-major
 // [page, nkv, Dv, slot].  Scores, the cap, the penalty, probabilities and sums are 32-bit.
 //
@@ -74,7 +79,7 @@ __global__ __launch_bounds__(kWave) void attn_softcap_simt_kernel(
     const T* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ positions, const int* __restrict__ slot_of_token, int nq, int nkv, int Dk, int Dv,
     int page_size, float scale, float cap, const void* __restrict__ r1, const void* __restrict__ r2, int r_dtype,
-    int window) {
+    int window, int chunk, const void* __restrict__ sink, int sink_dtype) {
   extern __shared__ float qs[];  // [Dk]
   const int t = blockIdx.x;
   const int h = blockIdx.y;
@@ -90,7 +95,8 @@ __global__ __launch_bounds__(kWave) void attn_softcap_simt_kernel(
   for (int d = lane; d < Dk; d += kWave) qs[d] = to_float(qr[d]);
   __syncthreads();
 
-  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  int first = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) first = max(first, pos / chunk * chunk);
   const int64_t k_page = static_cast<int64_t>(nkv) * page_size * Dk, v_page = static_cast<int64_t>(nkv) * page_size * Dv;
   const int64_t k_head = static_cast<int64_t>(kvh) * page_size * Dk, v_head = static_cast<int64_t>(kvh) * page_size * Dv;
 
@@ -136,11 +142,81 @@ __global__ __launch_bounds__(kWave) void attn_softcap_simt_kernel(
   }
 
   T* o = out + static_cast<int64_t>(t) * o_stride + h * Dv;
-  const float inv_l = 1.0f / l;
+  float keep = 1.0f;
+  if (sink) {  // one more term in the denominator, with no value behind it
+    const float sk = load_as_float(sink, sink_dtype, h);
+    const float m_all = fmaxf(m, sk);
+    keep = expf(m - m_all);
+    l = l * keep + expf(sk - m_all);
+  }
+  const float inv_l = keep / l;
 #pragma unroll
   for (int i = 0; i < kCapMaxD / kWave; ++i) {
     const int d = lane + i * kWave;
     if (d < Dv) o[d] = from_float<T>(acc[i] * inv_l);
+  }
+}
+
+// Operands of an attention that norms q and k over the whole projection.  One workgroup a (row, one of q, k, v):
+//   q <- q / rms(q) * wq  in place over all nq * Dk entries (wq null: q stays as it is);
+//   k likewise over all nkv * Dk entries, into the pages;
+//   v <- (1 - lambda) v + lambda v_first (v_first given), into the pages (d-major).
+// lambda is one number in memory, so that a captured launch reads the checkpoint's value.
+constexpr int kWideThreads = 256;
+template <typename T>
+__global__ __launch_bounds__(kWideThreads) void wide_norm_store_kernel(
+    T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride, const T* __restrict__ v,
+    long long v_stride, const T* __restrict__ v_first, long long vf_stride, const void* __restrict__ q_weight,
+    const void* __restrict__ k_weight, int w_dtype, const void* __restrict__ lambda, int lambda_dtype, float eps,
+    const int* __restrict__ positions, const int* __restrict__ slot_of_token, const int* __restrict__ block_table,
+    int table_stride, T* __restrict__ k_pages, T* __restrict__ v_pages, int nq, int nkv, int Dk, int Dv, int page_size) {
+  __shared__ float lds[kWideThreads / kWave];
+  const int64_t t = blockIdx.x;
+  const int what = blockIdx.y;
+  const int pos = positions[t];
+  if (what == 0) {
+    if (!q_weight) return;
+    const int width = nq * Dk;
+    T* row = q + t * q_stride;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += kWideThreads) {
+      const float x = to_float(row[i]);
+      ss = fmaf(x, x, ss);
+    }
+    const float inv = 1.0f / sqrtf(block_sum<kWideThreads / kWave>(ss, lds) / static_cast<float>(width) + eps);
+    for (int i = threadIdx.x; i < width; i += kWideThreads)
+      row[i] = from_float<T>(to_float(row[i]) * inv * load_as_float(q_weight, w_dtype, i));
+    return;
+  }
+  const int64_t page = block_table[static_cast<int64_t>(slot_of_token[t]) * table_stride + pos / page_size];
+  const int in_page = pos % page_size;
+  if (what == 1) {
+    const int width = nkv * Dk;
+    const T* row = k + t * k_stride;
+    float inv = 1.0f;
+    if (k_weight) {
+      float ss = 0.f;
+      for (int i = threadIdx.x; i < width; i += kWideThreads) {
+        const float x = to_float(row[i]);
+        ss = fmaf(x, x, ss);
+      }
+      inv = 1.0f / sqrtf(block_sum<kWideThreads / kWave>(ss, lds) / static_cast<float>(width) + eps);
+    }
+    for (int i = threadIdx.x; i < width; i += kWideThreads) {
+      const int g = i / Dk, d = i % Dk;
+      const float x = to_float(row[i]);
+      k_pages[((page * nkv + g) * page_size + in_page) * Dk + d] =
+          k_weight ? from_float<T>(x * inv * load_as_float(k_weight, w_dtype, i)) : row[i];
+    }
+    return;
+  }
+  const int width = nkv * Dv;
+  const float lam = v_first ? load_as_float(lambda, lambda_dtype, 0) : 0.f;
+  for (int i = threadIdx.x; i < width; i += kWideThreads) {
+    const int g = i / Dv, d = i % Dv;
+    T x = v[t * v_stride + i];
+    if (v_first) x = from_float<T>((1.0f - lam) * to_float(x) + lam * to_float(v_first[t * vf_stride + i]));
+    v_pages[((page * nkv + g) * Dv + d) * page_size + in_page] = x;
   }
 }
 
@@ -180,9 +256,11 @@ extern "C" int arle_attn_softcap_simt(const void* q, long long q_stride, void* o
                                       const void* k_pages, const void* v_pages, int dtype, const int* block_table,
                                       int table_stride, const int* positions, const int* slot_of_token, int tokens,
                                       int nq, int nkv, int Dk, int Dv, int page_size, float scale, float cap,
-                                      const void* r1, const void* r2, int r_dtype, int window, void* stream) {
+                                      const void* r1, const void* r2, int r_dtype, int window, int chunk,
+                                      const void* sink, int sink_dtype, void* stream) {
   if (tokens == 0) return 0;
-  if (Dk > kCapMaxD || Dv > kCapMaxD || nkv < 1 || nq % nkv != 0 || nq > 65535) return static_cast<int>(hipErrorInvalidValue);
+  if (Dk > kCapMaxD || Dv > kCapMaxD || nkv < 1 || nq % nkv != 0 || nq > 65535 || window < 0 || chunk < 0)
+    return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(tokens, nq);
   const size_t lds = static_cast<size_t>(Dk) * sizeof(float);
@@ -190,12 +268,41 @@ extern "C" int arle_attn_softcap_simt(const void* q, long long q_stride, void* o
     attn_softcap_simt_kernel<float><<<grid, kWave, lds, s>>>(
         static_cast<const float*>(q), q_stride, static_cast<float*>(out), o_stride, static_cast<const float*>(k_pages),
         static_cast<const float*>(v_pages), block_table, table_stride, positions, slot_of_token, nq, nkv, Dk, Dv,
-        page_size, scale, cap, r1, r2, r_dtype, window);
+        page_size, scale, cap, r1, r2, r_dtype, window, chunk, sink, sink_dtype);
   } else {
     attn_softcap_simt_kernel<bf16><<<grid, kWave, lds, s>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), o_stride, static_cast<const bf16*>(k_pages),
         static_cast<const bf16*>(v_pages), block_table, table_stride, positions, slot_of_token, nq, nkv, Dk, Dv,
-        page_size, scale, cap, r1, r2, r_dtype, window);
+        page_size, scale, cap, r1, r2, r_dtype, window, chunk, sink, sink_dtype);
+  }
+  return launch_status();
+}
+
+// q [T, nq*Dk] is normed in place over the whole row (q_weight [nq*Dk] or null); k [T, nkv*Dk] is normed likewise
+// (k_weight [nkv*Dk] or null) and goes to the pages; v [T, nkv*Dv], mixed with v_first by *lambda where v_first is
+// given, goes to the pages.
+extern "C" int arle_wide_norm_store(void* q, long long q_stride, const void* k, long long k_stride, const void* v,
+                                    long long v_stride, const void* v_first, long long vf_stride, int dtype,
+                                    const void* q_weight, const void* k_weight, int w_dtype, const void* lambda,
+                                    int lambda_dtype, float eps, const int* positions, const int* slot_of_token,
+                                    const int* block_table, int table_stride, void* k_pages, void* v_pages, int tokens,
+                                    int nq, int nkv, int Dk, int Dv, int page_size, void* stream) {
+  if (tokens == 0) return 0;
+  if (nq < 1 || nkv < 1 || Dk < 1 || Dv < 1 || page_size < 1 || (v_first && !lambda)) return static_cast<int>(hipErrorInvalidValue);
+  const dim3 grid(tokens, 3);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == kF32) {
+    wide_norm_store_kernel<float><<<grid, kWideThreads, 0, s>>>(
+        static_cast<float*>(q), q_stride, static_cast<const float*>(k), k_stride, static_cast<const float*>(v), v_stride,
+        static_cast<const float*>(v_first), vf_stride, q_weight, k_weight, w_dtype, lambda, lambda_dtype, eps, positions,
+        slot_of_token, block_table, table_stride, static_cast<float*>(k_pages), static_cast<float*>(v_pages), nq, nkv, Dk,
+        Dv, page_size);
+  } else {
+    wide_norm_store_kernel<bf16><<<grid, kWideThreads, 0, s>>>(
+        static_cast<bf16*>(q), q_stride, static_cast<const bf16*>(k), k_stride, static_cast<const bf16*>(v), v_stride,
+        static_cast<const bf16*>(v_first), vf_stride, q_weight, k_weight, w_dtype, lambda, lambda_dtype, eps, positions,
+        slot_of_token, block_table, table_stride, static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), nq, nkv, Dk,
+        Dv, page_size);
   }
   return launch_status();
 }
@@ -237,6 +344,8 @@ struct CapArgs {
   float scale, cap;
   const void* r1; const void* r2; int r_dtype;
   int window;
+  int chunk;                          // 0: none; else a row sees only the keys of its own chunk of so many positions
+  const void* sink; int sink_dtype;   // [nq] or null: exp(sink_h) joins the softmax's denominator
   int merge_floats;   // floats of dynamic LDS in front of the page ids
 };
 
@@ -283,8 +392,14 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
   // keys that any query of the item sees: from the first row's window to the last row's own position
   const int pos_lo = a.seg_start[seg] + (first_row - seg_first);
   const int pos_hi = a.seg_start[seg] + (last_row - seg_first);
-  const int key_lo = a.window > 0 ? max(0, pos_lo - a.window + 1) : 0;
-  const int my_lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  auto first_seen = [&](int p) {
+    int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    if (a.chunk > 0) lo = max(lo, p / a.chunk * a.chunk);
+    return lo;
+  };
+  const int key_lo = first_seen(pos_lo);
+  const int my_lo = first_seen(pos);
+  const float sink = a.sink ? load_as_float(a.sink, a.sink_dtype, head) : -INFINITY;
   const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
   const float pen1 = a.r1 ? load_as_float(a.r1, a.r_dtype, head) : 0.f;
   const float pen2 = a.r1 ? load_as_float(a.r2, a.r_dtype, head) : 0.f;
@@ -440,10 +555,10 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
       part_l[wave * 16 + n] = l_run;
     }
     __syncthreads();
-    float m_all = -INFINITY;
+    float m_all = sink;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) m_all = fmaxf(m_all, part_m[w * 16 + n]);
-    float l_all = 0.f, f[WAVES];
+    float l_all = a.sink ? __expf(sink - m_all) : 0.f, f[WAVES];
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
       f[w] = __expf(part_m[w * 16 + n] - m_all);
@@ -467,7 +582,11 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
     return;
   }
   if (!live) return;
-  const float inv_l = 1.0f / l_run;
+  float inv_l = 1.0f / l_run;
+  if (a.sink) {
+    const float m_all = fmaxf(m_run, sink), keep = __expf(m_run - m_all);
+    inv_l = keep / (l_run * keep + __expf(sink - m_all));
+  }
   bf16* orow = a.out + static_cast<int64_t>(row) * a.o_stride + head * a.Dv;
 #pragma unroll
   for (int c = 0; c < VC; ++c) {
@@ -492,20 +611,22 @@ extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* o
                                       int table_stride, const int* seg_row0, const int* seg_slot, const int* seg_start,
                                       int segments, int row_blocks, int heads_mode, int nq, int nkv, int Dk, int Dv,
                                       int page_size, float scale, float cap, const void* r1, const void* r2,
-                                      int r_dtype, int window, void* stream) {
+                                      int r_dtype, int window, int chunk, const void* sink, int sink_dtype,
+                                      void* stream) {
   if (segments == 0) return 0;
   if (Dk % 8 || Dk > 256 || Dv % 16 || Dv > 256 || page_size % 16 || nkv < 1 || nq % nkv || nq > 65535 ||
-      (heads_mode && nq / nkv > 16))
+      (heads_mode && nq / nkv > 16) || window < 0 || chunk < 0)
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const CapArgs a{static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), o_stride,
                   static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages), block_table, table_stride,
                   seg_row0, seg_slot, seg_start, segments, nq, nkv, Dk, Dv, page_size, scale, cap, r1, r2, r_dtype, window,
-                  heads_mode ? kCapSplitWaves * ((Dv / 16) * kWave * 4 + 32) : 0};
+                  chunk, sink, sink_dtype, heads_mode ? kCapSplitWaves * ((Dv / 16) * kWave * 4 + 32) : 0};
   // pages an item can see: its rows' windows (or everything the block table maps) and the tiles' rounding to 32 keys;
   // nothing of a step's lengths, so that a captured launch holds for every later step of its shape
   const long long mapped = static_cast<long long>(table_stride) * page_size;
-  const long long keys_seen = (window > 0 && window + 16 < mapped ? window + 16 : mapped) + 64;
+  const int span = window > 0 && chunk > 0 ? (window < chunk ? window : chunk) : (window > 0 ? window : chunk);
+  const long long keys_seen = (span > 0 && span + 16 < mapped ? span + 16 : mapped) + 64;
   const size_t page_bytes = (static_cast<size_t>(keys_seen) / page_size + 2) * sizeof(int);
   if (page_bytes > 48 * 1024) return static_cast<int>(hipErrorInvalidValue);
   const int size = (Dk + 1) / 2 > Dv ? (Dk + 1) / 2 : Dv;   // Dk counts half: a chunk of keys is 32 wide, of values 16

@@ -4,9 +4,15 @@
 //   reference counterpart: crates/cuda-kernels/csrc/misc/elementwise_basic.cu:186-211
 // silu_mul:     out[t, j] = silu(gate[t, j]) * up[t, j], silu(z) = z / (1 + exp(-z))
 //   reference counterpart: crates/cuda-kernels/csrc/misc/elementwise_basic.cu:18-24,34-95
+// tanh_cap:     x <- cap * tanh(x / cap) in place on float32 (soft-capped logits)
 #include "common.h"
 
 namespace arle {
+
+__global__ void tanh_cap_kernel(float* __restrict__ x, int64_t count, float cap, float inv_cap) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < count) x[i] = cap * tanhf(x[i] * inv_cap);
+}
 
 template <typename TT>
 __global__ void embed_gather_kernel(const TT* __restrict__ table, const int* __restrict__ ids,
@@ -164,5 +170,14 @@ extern "C" int arle_sum_partials(const float* parts, int n_parts, long long stri
     sum_partials_kernel<float><<<blocks, 256, 0, s>>>(parts, n_parts, stride, static_cast<float*>(out), count);
   else
     sum_partials_kernel<bf16><<<blocks, 256, 0, s>>>(parts, n_parts, stride, static_cast<bf16*>(out), count);
+  return launch_status();
+}
+
+// x float32 [count], in place.
+extern "C" int arle_tanh_cap(float* x, long long count, float cap, void* stream) {
+  if (count == 0) return 0;
+  if (!(cap > 0.f)) return static_cast<int>(hipErrorInvalidValue);
+  const unsigned blocks = static_cast<unsigned>((count + 255) / 256);
+  tanh_cap_kernel<<<blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(x, count, cap, 1.0f / cap);
   return launch_status();
 }

@@ -62,6 +62,7 @@ class StepBatch:
     kv_splits: int | None = None  # split-KV factor fixed by the caller (a captured graph), else chosen per call
     plan_token: int = 0          # names one pass over the layers (set by the model): what parts plan once a pass
     max_portion_kv: int = 0      # longest context (cached + new) among the segments of more than one token; 0: none
+    carry: dict = field(default_factory=dict)   # what a layer hands to later layers of the same pass (emptied by the model at the start of a pass)
 
 
 def packed_size(num_tokens: int, num_segments: int, num_wanted: int) -> int:

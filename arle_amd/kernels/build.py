@@ -39,6 +39,9 @@ SOURCES = {
     "polynorm": "polynorm.hip",
     "mlstm": "mlstm.hip",
     "attention_softcap": "attention_softcap.hip",
+    "post_norm": "post_norm.hip",
+    "latent": "latent.hip",
+    "moe": "moe.hip",
     "host": "host/runtime.cpp",
 }
 HEADERS = ("common.h", "attention_static.h", "attention_args.h", "attention_stream.h", "attention_portions.h",

@@ -1615,10 +1615,13 @@ def qkv_norm_store(q, k, v, *, num_q_heads: int, num_kv_heads: int, key_dim: int
 
 def attn_softcap_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_token, *, num_q_heads: int,
                       num_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
-                      softcap: float = 0.0, r1=None, r2=None, window: int = 0):
+                      softcap: float = 0.0, r1=None, r2=None, window: int = 0, chunk: int = 0, sink=None):
     """Causal attention of every row over its request's pages: scores scale (q . k), soft-capped (softcap > 0), less
-    r1_h ln(1 + r2_h distance) (r1, r2 [heads] given), over the last `window` keys (0: all)."""
-    _gpu(q, out, k_pages, v_pages, block_table, positions, slot_of_token, r1, r2)
+    r1_h ln(1 + r2_h distance) (r1, r2 [heads] given), over the last `window` keys (0: all) and, with `chunk` > 0,
+    over the keys of the row's own chunk of so many positions only; `sink` [heads]: exp(sink_h) joins the softmax's
+    denominator."""
+    _gpu(q, out, k_pages, v_pages, block_table, positions, slot_of_token, r1, r2, sink)
+    _check_sink(sink, num_q_heads, window, chunk)
     tokens = q.shape[0]
     _rows(q, "q")
     _rows(out, "out")
@@ -1638,8 +1641,20 @@ def attn_softcap_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_
     lib.call("arle_attn_softcap_simt", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(),
              v_pages.data_ptr(), _code(q), block_table.data_ptr(), block_table.shape[1], positions.data_ptr(),
              slot_of_token.data_ptr(), tokens, num_q_heads, num_kv_heads, key_dim, value_dim, page_size, float(scale),
-             float(softcap), _ptr(r1), _ptr(r2), _code(r1) if r1 is not None else 0, int(window), _stream())
+             float(softcap), _ptr(r1), _ptr(r2), _code(r1) if r1 is not None else 0, int(window), int(chunk), _ptr(sink),
+             _code(sink) if sink is not None else 0, _stream())
     return out
+
+
+def _check_sink(sink, num_q_heads: int, window: int, chunk: int) -> None:
+    _need(window >= 0 and chunk >= 0, "a window and a chunk size are not negative")
+    if sink is not None:
+        _need(sink.shape == (num_q_heads,) and sink.is_contiguous() and sink.dtype in _CODES, "sink must be [heads]")
+
+
+def mask_span(window: int, chunk: int) -> int:
+    """The most keys a row sees under a window and a chunk size (0 for either: none); 0: all earlier keys."""
+    return min(window, chunk) if window > 0 and chunk > 0 else max(window, chunk)
 
 
 CAP_MFMA_MAX_DIM = 256
@@ -1661,10 +1676,11 @@ def attn_softcap_mfma_fits(window: int, table_width: int, page_size: int) -> boo
 
 def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *, max_qlen: int,
                       num_q_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
-                      softcap: float = 0.0, r1=None, r2=None, window: int = 0):
+                      softcap: float = 0.0, r1=None, r2=None, window: int = 0, chunk: int = 0, sink=None):
     """`attn_softcap_simt` on the matrix cores, bfloat16: sixteen rows of a segment a wave, or (when every segment is
     one decoded row and a kv head has at most sixteen q heads) one row's q heads of a kv head a wave."""
-    _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, r1, r2)
+    _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, r1, r2, sink)
+    _check_sink(sink, num_q_heads, window, chunk)
     tokens = q.shape[0]
     _rows(q, "q")
     _rows(out, "out")
@@ -1686,7 +1702,7 @@ def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot,
     if r1 is not None:
         _need(r1.shape == (num_q_heads,) and r2.shape == (num_q_heads,) and r1.dtype == r2.dtype and r1.dtype in _CODES
               and r1.is_contiguous() and r2.is_contiguous(), "r1, r2 must be [heads] of one type")
-    _need(attn_softcap_mfma_fits(window, block_table.shape[1], page_size),
+    _need(attn_softcap_mfma_fits(mask_span(window, chunk), block_table.shape[1], page_size),
           "the keys a row sees span more pages than the kernel holds ids for")
     heads_mode = max_qlen == 1 and group <= 16 and segments == tokens
     row_blocks = tokens // 16 + segments      # no fewer than the sixteen-row blocks of all segments together
@@ -1694,5 +1710,193 @@ def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot,
              v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], seg_row0.data_ptr(), seg_slot.data_ptr(),
              seg_start.data_ptr(), segments, row_blocks, 1 if heads_mode else 0, num_q_heads, num_kv_heads, key_dim,
              value_dim, page_size, float(scale), float(softcap), _ptr(r1), _ptr(r2),
-             _code(r1) if r1 is not None else 0, int(window), _stream())
+             _code(r1) if r1 is not None else 0, int(window), int(chunk), _ptr(sink),
+             _code(sink) if sink is not None else 0, _stream())
+    return out
+
+
+def wide_norm_store(q, k, v, *, num_q_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, eps: float,
+                    q_weight=None, k_weight=None, v_first=None, mix=None, positions, slot_of_token, block_table,
+                    k_pages, v_pages, page_size: int):
+    """RMS norm of q over its whole row (in place, weight [heads * Dk]) and of k over its whole row (weight
+    [kv heads * Dk]); k goes to the pages, and so does v, as (1 - mix) v + mix v_first where v_first [T, kv heads * Dv]
+    is given (`mix`: a tensor of one number)."""
+    _gpu(q, k, v, q_weight, k_weight, v_first, mix, positions, slot_of_token, block_table, k_pages, v_pages)
+    tokens = q.shape[0]
+    for name, t, width in (("q", q, num_q_heads * key_dim), ("k", k, num_kv_heads * key_dim),
+                           ("v", v, num_kv_heads * value_dim)):
+        _rows(t, name)
+        _need(t.shape == (tokens, width) and t.dtype == q.dtype and t.dtype in _CODES, f"{name} must be [T, {width}]")
+    w_code = 0
+    for w, width in ((q_weight, num_q_heads * key_dim), (k_weight, num_kv_heads * key_dim)):
+        if w is not None:
+            _need(w.shape == (width,) and w.is_contiguous() and w.dtype in _CODES, "a whole-row norm weight spans the row")
+            w_code = _code(w)
+    if q_weight is not None and k_weight is not None:
+        _need(q_weight.dtype == k_weight.dtype, "q and k norm weights must be of one type")
+    if v_first is not None:
+        _rows(v_first, "v_first")
+        _need(v_first.shape == v.shape and v_first.dtype == v.dtype, "v_first must match v")
+        _need(mix is not None and mix.numel() == 1 and mix.dtype in _CODES, "the mixing weight is one number")
+    _check_kv_pages(k_pages, v_pages, num_kv_heads, page_size, key_dim, value_dim, q.dtype)
+    _i32(positions, "positions", tokens)
+    _i32(slot_of_token, "slot_of_token", tokens)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [slots, pages]")
+    lib.call("arle_wide_norm_store", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+             _ptr(v_first), v_first.stride(0) if v_first is not None else 0, _code(q), _ptr(q_weight), _ptr(k_weight),
+             w_code, _ptr(mix) if v_first is not None else 0, _code(mix) if v_first is not None else 0, float(eps),
+             positions.data_ptr(), slot_of_token.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+             k_pages.data_ptr(), v_pages.data_ptr(), tokens, num_q_heads, num_kv_heads, key_dim, value_dim,
+             int(page_size), _stream())
+
+
+# ------------------------------------------------------------------ a norm on a sublayer's output
+
+NORM_ADD_MAX_WIDTH = 16384
+
+
+def _addend_args(term, rows: int, width: int):
+    """(pointer, parts, part stride, row stride, type code, weights pointer) of one addend of `norm_add`: a tensor
+    [T, W]; a float32 stack [S, T, W] of partial sums; or (outputs [T, n, W], weights float32 [T, n])."""
+    if term is None:
+        return (0, 0, 0, 0, 0, 0)
+    if isinstance(term, tuple):
+        outs, weights = term
+        _need(outs.dim() == 3 and outs.shape[0] == rows and outs.shape[2] == width and outs.is_contiguous()
+              and outs.dtype in _CODES, "weighted outputs must be contiguous [T, n, W]")
+        _need(weights.shape == outs.shape[:2] and weights.dtype == torch.float32 and weights.is_contiguous(),
+              "their weights must be contiguous float32 [T, n]")
+        return (outs.data_ptr(), outs.shape[1], width, outs.shape[1] * width, _code(outs), weights.data_ptr())
+    _need(term.dim() in (2, 3) and tuple(term.shape[-2:]) == (rows, width) and term.is_contiguous() and term.dtype in _CODES,
+          "an addend must match the residual ([T, W] or a float32 stack [S, T, W])")
+    _need(term.dim() == 2 or (term.dtype == torch.float32 and term.shape[0] >= 1), "a stack of partial sums is float32")
+    return (term.data_ptr(), term.shape[0] if term.dim() == 3 else 1, rows * width, width, _code(term), 0)
+
+
+def norm_add(residual: torch.Tensor, terms, weight: torch.Tensor, eps: float, *, one_plus: bool = False,
+             act_dtype: torch.dtype | None = None):
+    """residual += y / sqrt(mean(y^2) + eps) * weight (or 1 + weight) for y the sum of up to two `terms`, in place;
+    returns the updated residual rounded to `act_dtype` (None: nothing is returned)."""
+    terms = [t for t in (terms if isinstance(terms, list) else [terms]) if t is not None]
+    _need(1 <= len(terms) <= 2, "norm_add takes one or two addends")
+    _gpu(residual, weight, *[x for t in terms for x in (t if isinstance(t, tuple) else (t,))])
+    _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
+          "residual must be contiguous float32 [T, W]")
+    rows, width = residual.shape
+    _need(0 < width <= NORM_ADD_MAX_WIDTH, f"norm_add takes widths up to {NORM_ADD_MAX_WIDTH}")
+    _need(weight.shape == (width,) and weight.is_contiguous() and weight.dtype in _CODES, "norm weight must be [width]")
+    act = torch.empty((rows, width), dtype=act_dtype, device=residual.device) if act_dtype is not None else None
+    args = []
+    for i in range(2):
+        args += _addend_args(terms[i] if i < len(terms) else None, rows, width)
+    lib.call("arle_norm_add", residual.data_ptr(), *args, weight.data_ptr(), _code(weight), 1 if one_plus else 0,
+             _ptr(act), _code(act) if act is not None else 0, rows, width, float(eps), _stream())
+    return act
+
+
+def tanh_cap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap tanh(x / cap) in place on contiguous float32."""
+    _gpu(x)
+    _need(x.dtype == torch.float32 and x.is_contiguous() and cap > 0, "tanh_cap_ takes contiguous float32 and a positive cap")
+    lib.call("arle_tanh_cap", x.data_ptr(), x.numel(), float(cap), _stream())
+    return x
+
+
+# ------------------------------------------------------------------ latent attention's operands
+
+HEAD_PROJ_MAX_K = 2048
+
+
+def latent_prep(q, dkv, q_full, *, heads: int, dim: int, rot_dim: int, rank: int, c_weight, eps: float, cos, sin,
+                rotary_dims: int, positions, slot_of_token, block_table, k_pages, v_pages, page_size: int):
+    """dkv [T, rank + rot_dim]: the first `rank` entries RMS-normed (c), the rest rotated (interleaved pairs over the
+    first `rotary_dims`), [c | k_rot] to the key pages and c to the value pages; the rotated part of every head of
+    q [T, heads * (dim + rot_dim)] goes, rotated, to the last rot_dim entries of its head in
+    q_full [T, heads * (rank + rot_dim)]."""
+    _gpu(q, dkv, q_full, c_weight, cos, sin, positions, slot_of_token, block_table, k_pages, v_pages)
+    tokens = q.shape[0]
+    for name, t, width in (("q", q, heads * (dim + rot_dim)), ("dkv", dkv, rank + rot_dim),
+                           ("q_full", q_full, heads * (rank + rot_dim))):
+        _rows(t, name)
+        _need(t.shape == (tokens, width) and t.dtype == q.dtype and t.dtype in _CODES, f"{name} must be [T, {width}]")
+    _need(c_weight.shape == (rank,) and c_weight.is_contiguous() and c_weight.dtype in _CODES, "the latent's norm weight must be [rank]")
+    _need(0 <= rotary_dims <= rot_dim and rotary_dims % 2 == 0, "rotary dims must be even and within the rotated part")
+    if rotary_dims:
+        for name, t in (("cos", cos), ("sin", sin)):
+            _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rotary_dims // 2 and t.is_contiguous(),
+                  f"{name} must be contiguous float32 [positions, rotary_dims / 2]")
+    _check_kv_pages(k_pages, v_pages, 1, page_size, rank + rot_dim, rank, q.dtype)
+    _i32(positions, "positions", tokens)
+    _i32(slot_of_token, "slot_of_token", tokens)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [slots, pages]")
+    lib.call("arle_latent_prep", q.data_ptr(), q.stride(0), dkv.data_ptr(), dkv.stride(0), q_full.data_ptr(),
+             q_full.stride(0), _code(q), c_weight.data_ptr(), _code(c_weight), float(eps), _ptr(cos), _ptr(sin),
+             int(rotary_dims), positions.data_ptr(), slot_of_token.data_ptr(), block_table.data_ptr(),
+             block_table.shape[1], k_pages.data_ptr(), v_pages.data_ptr(), tokens, heads, dim, rot_dim, rank,
+             int(page_size), _stream())
+
+
+def head_proj(x, wt, out, *, heads: int, in_head: int, out_head: int):
+    """out[t, h * out_head + n] = sum_k x[t, h * in_head + k] wt[h, k, n] for wt [heads, K, N]: a matrix of its own
+    for every head, one fixed-order chain over k an output."""
+    _gpu(x, wt, out)
+    _rows(x, "x")
+    _rows(out, "out")
+    _need(wt.dim() == 3 and wt.shape[0] == heads and wt.is_contiguous(), "wt must be contiguous [heads, K, N]")
+    K, N = wt.shape[1], wt.shape[2]
+    _need(x.dtype == wt.dtype == out.dtype and x.dtype in _CODES, "x, wt and out must be of one type")
+    _need(K <= HEAD_PROJ_MAX_K, f"head_proj takes inner sizes up to {HEAD_PROJ_MAX_K}")
+    _need(x.shape[0] == out.shape[0] and (heads - 1) * in_head + K <= x.shape[1]
+          and (heads - 1) * out_head + N <= out.shape[1], "a head's numbers must lie inside its row")
+    lib.call("arle_head_proj", x.data_ptr(), x.stride(0), int(in_head), wt.data_ptr(), out.data_ptr(), out.stride(0),
+             int(out_head), _code(x), x.shape[0], heads, K, N, _stream())
+    return out
+
+
+# ------------------------------------------------------------------ mixture of experts
+
+MOE_MAX_EXPERTS = 1024
+MOE_MAX_TOP = 64
+
+
+def moe_route(x, router, correction, *, top: int, scale: float):
+    """(ids int32 [T, top], weights float32 [T, top]) of a sigmoid router: z = router x in 32-bit sums,
+    s = sigmoid(z), the `top` largest s + correction chosen (ties: the lower index), weights s / (sum + 1e-20) * scale
+    in the order they were chosen."""
+    _gpu(x, router, correction)
+    _rows(x, "x")
+    experts, width = router.shape
+    _need(router.dim() == 2 and router.is_contiguous() and router.dtype in _CODES and x.shape[1] == width and x.dtype in _CODES,
+          "router must be contiguous [experts, width]")
+    _need(1 <= top <= min(experts, MOE_MAX_TOP) and experts <= MOE_MAX_EXPERTS,
+          f"the router takes up to {MOE_MAX_EXPERTS} experts and {MOE_MAX_TOP} choices a token")
+    if correction is not None:
+        _need(correction.shape == (experts,) and correction.is_contiguous() and correction.dtype in _CODES,
+              "correction must be [experts]")
+    ids = torch.empty((x.shape[0], top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((x.shape[0], top), dtype=torch.float32, device=x.device)
+    lib.call("arle_moe_route", x.data_ptr(), x.stride(0), _code(x), router.data_ptr(), _code(router), _ptr(correction),
+             _code(correction) if correction is not None else 0, ids.data_ptr(), weights.data_ptr(), x.shape[0], width,
+             experts, int(top), float(scale), _stream())
+    return ids, weights
+
+
+def moe_expert(x, w, ids, *, gate_up: bool):
+    """The chosen experts' products.  gate_up: x [T, K], w [experts, 2N, K] (gate rows, then up rows) ->
+    silu(gate) * up as [T * top, N] of x's type, row t * top + k for token t's k-th choice.  Else: x [T * top, K],
+    w [experts, N, K] -> float32 [T * top, N]."""
+    _gpu(x, w, ids)
+    _rows(x, "x")
+    _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.is_contiguous(), "ids must be contiguous int32 [T, top]")
+    tokens, top = ids.shape
+    _need(w.dim() == 3 and w.is_contiguous() and w.dtype == x.dtype and x.dtype in _CODES and w.shape[2] == x.shape[1],
+          "w must be contiguous [experts, N, K] of x's type")
+    _need(x.shape[0] == (tokens if gate_up else tokens * top), "x has a row a token (gate|up) or a row a choice (down)")
+    _need(not gate_up or w.shape[1] % 2 == 0, "gate|up has an even number of rows")
+    N = w.shape[1] // 2 if gate_up else w.shape[1]
+    out = torch.empty((tokens * top, N), dtype=x.dtype if gate_up else torch.float32, device=x.device)
+    lib.call("arle_moe_expert", x.data_ptr(), x.stride(0), w.data_ptr(), ids.data_ptr(), out.data_ptr(), _code(x),
+             1 if gate_up else 0, tokens, w.shape[0], top, N, x.shape[1], _stream())
     return out

@@ -12,8 +12,8 @@ import sys
 
 from ..kernels import ops
 from ..parts import base  # noqa: F401  (registries)
-from ..parts import (attention, block, embedding, feed_forward, mlstm, norm, position,  # noqa: F401  registers the stock parts
-                     short_conv, softcap_attention)
+from ..parts import (attention, block, embedding, feed_forward, latent_attention, mlstm, moe, norm,  # noqa: F401  registers the stock parts
+                     position, short_conv, softcap_attention, wide_norm_attention)
 from ..parts.base import Runtime, build_part, expected_tensors, lookup
 from ..parts.spec import ModelSpec
 
@@ -150,6 +150,7 @@ class DecoderModel:
         # every pass over the layers gets a name of its own (a pass that is being captured into a graph too: its
         # first layer has to plan inside the graph): parts that prepare something once a step key it with this
         batch.plan_token = ops.new_plan_token()
+        batch.carry = {}     # what layers hand to later layers lives for one pass
         residual = self.embedding.forward(batch.token_ids)
         delta = None
         dump = os.environ.get(DEBUG_DUMP_ENV) is not None

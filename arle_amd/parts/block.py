@@ -30,6 +30,46 @@ class PreNormBlock:
         return residual, self.feed_forward.forward(b)
 
 
+@register("block", "post_norm")
+class PostNormBlock:
+    """h += norm_a(mixer(h)); h += norm_b(ffn(h)): the sublayers read the residual itself, the norms stand on their
+    outputs.  norm roles: "mixer_out", "ffn_out" (the second only with a feed-forward).  The residual is float32;
+    what a sublayer reads is the residual in the activation type, which the norm's kernel writes beside the sum it
+    updates (`add_into`), and which goes from block to block in `batch.carry`.  Nothing is left for the next block
+    to add."""
+
+    norm_roles = ("mixer_out", "ffn_out")
+    CARRY = "residual_rounded"     # batch.carry[CARRY] = (the residual tensor, its copy in the activation type)
+
+    def __init__(self, mixer, feed_forward, norms: dict):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norms = norms
+        self.norm_mixer = norms.get("mixer_out") if mixer is not None else None
+        self.norm_ffn = norms.get("ffn_out") if feed_forward is not None else None
+
+    def _reads(self, residual, batch):
+        kept = batch.carry.get(self.CARRY)
+        if kept is not None and kept[0] is residual:
+            return kept[1]
+        act = next(iter(self.norms.values())).rt.act_dtype
+        if act == residual.dtype:
+            return residual
+        from ..kernels import ops
+        return ops.sum_partials(residual.unsqueeze(0), act)     # one part: a rounding pass
+
+    def forward(self, residual, delta, batch, cache_view):
+        if delta is not None:
+            raise ValueError("a post_norm block stands behind blocks that leave nothing to add")
+        x = self._reads(residual, batch)
+        if self.mixer is not None:
+            x = self.norm_mixer.add_into(residual, self.mixer.forward(x, batch, cache_view))
+        if self.feed_forward is not None:
+            x = self.norm_ffn.add_into(residual, self.feed_forward.forward(x))
+        batch.carry[self.CARRY] = (residual, x)
+        return residual, None
+
+
 @register("block", "parallel")
 class ParallelBlock:
     """h += mixer(norm_a(h)) + ffn(norm_b(h)): both read the same residual.  norm roles: "mixer_in", "ffn_in" (the

@@ -33,7 +33,8 @@ class TokenEmbedding(Part):
 
 @register("head", "linear")
 class LinearHead(Part):
-    """params: vocab_size, hidden_size.  Logits are float32."""
+    """params: vocab_size, hidden_size, softcap (0 or absent: none; else logits <- cap tanh(logits / cap)).
+    Logits are float32."""
 
     graph_safe = True  # launches depend on shapes only, never on the values of a step
 
@@ -44,6 +45,7 @@ class LinearHead(Part):
     def __init__(self, params, tensors, rt, children=None):
         super().__init__(params, tensors, rt, children)
         self.proj = Linear(tensors["weight"], rt.weight_tiles)
+        self.softcap = float(params.get("softcap") or 0.0)
 
     def products(self):
         if self.proj.weight.dtype != torch.bfloat16:
@@ -51,4 +53,7 @@ class LinearHead(Part):
         return [("head", self.proj.out_features, self.proj.in_features, False, None)]
 
     def forward(self, x):
-        return self.proj(x, out_dtype=torch.float32)
+        logits = self.proj(x, out_dtype=torch.float32)
+        if self.softcap > 0.0 and logits.numel():
+            logits = ops.tanh_cap_(logits.contiguous(), self.softcap)
+        return logits

@@ -16,7 +16,8 @@ from .linear import Linear
 
 @register("feed_forward", "swiglu")
 class SwiGLU(Part):
-    """params: hidden_size, intermediate_size."""
+    """params: hidden_size, intermediate_size, float32_out (bool, default False: the down projection hands on its
+    32-bit sums instead of rounding them to the activation type)."""
 
     graph_safe = True  # launches depend on shapes only, never on the values of a step
 
@@ -28,6 +29,7 @@ class SwiGLU(Part):
     def __init__(self, params, tensors, rt, children=None):
         super().__init__(params, tensors, rt, children)
         self.inter = int(params["intermediate_size"])
+        self.float32_out = bool(params.get("float32_out", False))
         gate, up = tensors["gate"], tensors["up"]
         if gate.dtype != up.dtype:
             raise ValueError("gate and up projections must be stored in one type")
@@ -56,7 +58,7 @@ class SwiGLU(Part):
         else:
             gu = self.gate_up(x)
             act = ops.silu_mul(gu[:, : self.inter], gu[:, self.inter:])
-        return self.down(act, partials_ok=True)
+        return self.down(act, out_dtype=torch.float32 if self.float32_out else None, partials_ok=True)
 
 
 @register("feed_forward", "polynorm")

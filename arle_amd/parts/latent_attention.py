@@ -1,0 +1,112 @@
+"""Latent attention: every token caches one compressed vector c and one rotated key part shared by all heads.
+
+Per token, with h the mixer's input, H heads, per head D unrotated and R rotated query/key entries, value size Dv,
+latent size C:
+
+    q = W_q h, head by head [D unrotated | R rotated];     W_dkv h = [C entries | R entries]
+    c = rms_norm(first C entries) * w_c;                    k_rot = rotate(last R entries)        (one for all heads)
+    k_h = W_uk,h c,  v_h = W_uv,h c
+    s_ij,h = scale (q_h,i . k_h,j + rotate(q_rot,h,i) . k_rot,j)    for 0 <= i - j < window  (None: every j <= i)
+    p = exp(s) / (sum_j exp(s_ij) + exp(sink_h))            (sink: a learned number a head, optional)
+    out = W_o concat_h(sum_j p_j v_h,j)
+
+The maps W_uk and W_uv are folded into the query and the output: q'_h = W_uk,h^T q_h, so that
+s = scale (q'_h . c + q_rot . k_rot), and out_h = W_uv,h (sum_j p_j c_j).  The attention is then one of H query heads
+over a single key/value head with keys [c | k_rot] and values c, which is what the pages hold
+(`[1, page, C + R]`, and c once more d-major `[1, C, page]` as the second operand of the matrix cores); keys and
+values of the heads are never formed.  The rotation is a position part (`rope_interleaved`) whose table the
+preparation kernel reads.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache.manager import PAGE, PagedNeed, PageTensor
+from ..kernels import ops
+from .base import Part, WeightDecl, register
+from .linear import Linear
+from .softcap_attention import softcap_attention
+
+
+@register("mixer", "latent_attention")
+class LatentAttention(Part):
+    """params: hidden_size, heads, dim, rot_dim, value_dim, rank, eps, scale, window (int | None), sink (bool),
+    position (PartSpec of the rotation over the rot_dim part)."""
+
+    graph_safe = True  # positions, slots and lengths are read on the GPU; launches depend on shapes only
+
+    @classmethod
+    def declare_weights(cls, params):
+        h, H = params["hidden_size"], params["heads"]
+        D, R, Dv, C = params["dim"], params["rot_dim"], params["value_dim"], params["rank"]
+        decl = {"q": WeightDecl((H * (D + R), h)), "dkv": WeightDecl((C + R, h)), "c_norm": WeightDecl((C,), init="ones"),
+                "uk": WeightDecl((H * D, C)), "uv": WeightDecl((H * Dv, C)), "o": WeightDecl((h, H * Dv))}
+        if params.get("sink"):
+            decl["sink"] = WeightDecl((H,), init="normal")
+        return decl
+
+    @classmethod
+    def children(cls, params):
+        return {"position": ("position", params["position"])}
+
+    @classmethod
+    def declare_cache(cls, params):
+        C, R = int(params["rank"]), int(params["rot_dim"])
+        return PagedNeed(window=params.get("window"),
+                         tensors=(PageTensor("k", (1, PAGE, C + R)), PageTensor("v", (1, C, PAGE))))
+
+    def cache_need(self):
+        return self.declare_cache(self.params)
+
+    def __init__(self, params, tensors, rt, children=None):
+        super().__init__(params, tensors, rt, children)
+        self.H, self.D, self.R = int(params["heads"]), int(params["dim"]), int(params["rot_dim"])
+        self.Dv, self.C = int(params["value_dim"]), int(params["rank"])
+        if not (0 < self.C + self.R <= ops.MAX_HEAD_DIM):
+            raise ValueError(f"latent and rotated sizes {self.C} + {self.R} are not supported: the attention kernels "
+                             f"take keys of 1..{ops.MAX_HEAD_DIM}")
+        if max(self.D, self.C) > ops.HEAD_PROJ_MAX_K:
+            raise ValueError(f"head and latent sizes up to {ops.HEAD_PROJ_MAX_K} are taken")
+        self.eps = float(params.get("eps", 0.0))
+        self.scale = float(params["scale"])
+        self.window = int(params.get("window") or 0)
+        self.position = children["position"]
+        wq, wd = tensors["q"], tensors["dkv"]
+        if len({wq.dtype, wd.dtype, tensors["uk"].dtype, tensors["uv"].dtype}) != 1:
+            raise ValueError("the projections of a latent attention must be stored in one type")
+        self.q_width = self.H * (self.D + self.R)
+        self.proj = Linear(torch.cat([wq, wd], dim=0).contiguous(), rt.weight_tiles)
+        self.c_norm = tensors["c_norm"]
+        # a matrix a head, stored [inner, outer]: q'_h = q_h W_uk,h (W_uk,h is [D, C] as it lies), out_h = lat_h W_uv,h^T
+        self.uk = tensors["uk"].view(self.H, self.D, self.C)
+        self.uv_t = tensors["uv"].view(self.H, self.Dv, self.C).transpose(1, 2).contiguous()
+        self.sink = tensors.get("sink")
+        self.o = Linear(tensors["o"], rt.weight_tiles)
+
+    def products(self):
+        if self.proj.weight.dtype != torch.bfloat16:
+            return []
+        return [("q_dkv", self.proj.out_features, self.proj.in_features, False, None),
+                ("o", self.o.out_features, self.o.in_features, False, "norm")]
+
+    def forward(self, x, batch, cache):
+        """x [T, H] -> float32 [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
+        if not cache.writes:
+            raise ValueError("a latent attention keeps a cache of its own")
+        H, D, R, C, Dv = self.H, self.D, self.R, self.C, self.Dv
+        self.position.ensure_positions(batch.max_position + 1)
+        cos, sin, rot = self.position.fused_rotary()
+        y = self.proj(x)
+        q, dkv = y[:, :self.q_width], y[:, self.q_width:]
+        q_full = torch.empty((x.shape[0], H * (C + R)), dtype=x.dtype, device=x.device)
+        ops.latent_prep(q, dkv, q_full, heads=H, dim=D, rot_dim=R, rank=C, c_weight=self.c_norm, eps=self.eps, cos=cos,
+                        sin=sin, rotary_dims=rot, positions=batch.positions, slot_of_token=batch.slot_of_token,
+                        block_table=cache.block_table, k_pages=cache.pages["k"], v_pages=cache.pages["v"],
+                        page_size=cache.page_size)
+        ops.head_proj(q, self.uk, q_full, heads=H, in_head=D + R, out_head=C + R)
+        latent = torch.empty((x.shape[0], H * C), dtype=x.dtype, device=x.device)
+        softcap_attention(q_full, latent, cache, batch, num_q_heads=H, num_kv_heads=1, key_dim=C + R, value_dim=C,
+                          scale=self.scale, softcap=0.0, r1=None, r2=None, window=self.window, sink=self.sink)
+        heads_out = torch.empty((x.shape[0], H * Dv), dtype=x.dtype, device=x.device)
+        ops.head_proj(latent, self.uv_t, heads_out, heads=H, in_head=C, out_head=Dv)
+        return self.o(heads_out, out_dtype=torch.float32, partials_ok=True)   # into the 32-bit residual unrounded

@@ -12,22 +12,38 @@ from .base import Part, WeightDecl, register
 
 @register("norm", "rmsnorm")
 class RMSNorm(Part):
-    """params: width, eps."""
+    """params: width, eps, one_plus (bool, default False: the checkpoint stores the weight around zero and the norm
+    multiplies by 1 + w; the sum is formed in 32 bits, where it is exact or rounded once).
+
+    Beside the norm of the residual (`forward`, `add_norm`) it can stand on a sublayer's output: `add_into` norms
+    what the sublayer left and adds the result into the residual."""
 
     graph_safe = True  # launches depend on shapes only, never on the values of a step
 
     @classmethod
     def declare_weights(cls, params):
-        return {"weight": WeightDecl((params["width"],), init="ones")}
+        return {"weight": WeightDecl((params["width"],), init="near_zero" if params.get("one_plus") else "ones")}
 
     def __init__(self, params, tensors, rt, children=None):
         super().__init__(params, tensors, rt, children)
-        self.weight = tensors["weight"]
+        self.one_plus = bool(params.get("one_plus", False))
+        self.stored = tensors["weight"]
+        self.weight = (1.0 + self.stored.float()) if self.one_plus else self.stored
         self.eps = float(params["eps"])
         self.width = int(params["width"])
 
     def forward(self, x, rows=None):
         return ops.rmsnorm(x, self.weight, self.eps, self.rt.act_dtype, rows=rows)
+
+    def add_into(self, residual, terms, want_rounded: bool = True):
+        """residual (float32, in place) += norm(sum of `terms`): one or two of a tensor [T, W], a float32 stack
+        [S, T, W] of partial sums, or (outputs [T, n, W], float32 weights [T, n]).  Returns the updated residual in
+        the activation type: itself in a float32 engine, else a rounded copy from the same pass (None if not
+        wanted)."""
+        rounded = want_rounded and self.rt.act_dtype != residual.dtype
+        out = ops.norm_add(residual, terms, self.stored, self.eps, one_plus=self.one_plus,
+                           act_dtype=self.rt.act_dtype if rounded else None)
+        return out if rounded else residual
 
     def add_norm(self, residual, delta, rows=None):
         """residual (float32) += delta, then the norm of it; delta None: just the norm."""

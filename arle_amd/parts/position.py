@@ -5,6 +5,8 @@
 pairs (i, i + rotary_dim/2).  infer/src/weight_loader.rs:955-989 builds the same table
 (and then narrows it to bf16, which this engine does not: angles, cos and sin stay
 32-bit); rotation as crates/cuda-kernels/csrc/attention/prefill_attention_paged_prep.cu:60-76.
+`rope_interleaved`: the same angles with entry 2i paired with entry 2i + 1; it only keeps the table, which the
+kernel of the mixer that names it applies.
 `none`: no position encoding.
 """
 from __future__ import annotations
@@ -71,6 +73,19 @@ class RopeNeox(Part):
         ops.qk_prep(q, k, k, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads,
                     head_dim=self.head_dim, eps=0.0, cos=self.cos, sin=self.sin,
                     rotary_dim=self.rotary_dim, positions=positions)
+
+
+@register("position", "rope_interleaved")
+class RopeInterleaved(RopeNeox):
+    """params: head_dim (size of the vector that is rotated), rotary_dim (its first entries that rotate; default all),
+    theta, max_positions.  The pair (u, v) = (x[2i], x[2i+1]) at position p becomes (u cos a - v sin a,
+    v cos a + u sin a), a = p theta^(-2i/rotary_dim).  The q/k preparation of the rotate-half layout does not know
+    this pairing, so `fusable` is False and `apply` refuses: a mixer reads `fused_rotary()` and rotates itself."""
+
+    fusable = False
+
+    def apply(self, q, k, positions, num_q_heads, num_kv_heads):
+        raise NotImplementedError("rope_interleaved is applied by the kernels of the mixer that names it")
 
 
 @register("position", "none")

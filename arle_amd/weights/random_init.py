@@ -39,8 +39,16 @@ def _init_zeros(shape, gen, std, norm_std, device):
     return torch.zeros(shape, dtype=torch.float32, device=device)
 
 
+def _init_near_zero(shape, gen, std, norm_std, device):
+    """A norm weight that is stored around zero (the norm multiplies by 1 + w): N(0, norm_std)."""
+    t = torch.zeros(shape, dtype=torch.float32, device=device)
+    if norm_std:
+        t += torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * norm_std
+    return t
+
+
 # WeightDecl.init -> how a random tensor of that kind is filled: f(shape, generator, std, norm_std, device) -> float32
-INITS = {"normal": _init_normal, "ones": _init_ones, "zeros": _init_zeros}
+INITS = {"normal": _init_normal, "ones": _init_ones, "zeros": _init_zeros, "near_zero": _init_near_zero}
 
 
 def register_init(name: str, fill) -> None:
