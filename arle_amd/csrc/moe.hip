@@ -9,7 +9,7 @@
 // step sorts anything and a launch's shape follows the number of rows alone.  The result of (token t, its k-th
 // choice) lies at row t * top + k: the gate|up pass leaves the activation there, the down pass the expert's output,
 // which the consumer weighs and adds in the order of k.  Every output is summed in one fixed order over K (chains
-// of 16, added in ascending order), whatever else the step holds.
+// of 16, added in ascending order), whatever else the step holds.  bfloat16 runs the matrix-core form further down.
 #include "common.h"
 
 namespace arle {
@@ -197,6 +197,115 @@ __global__ __launch_bounds__(kExpertThreads) void moe_expert_kernel(const T* __r
   }
 }
 
+// ---- matrix-core form (bfloat16) -----------------------------------------------------------------
+// A workgroup of four waves takes one expert, 256 consecutive rows of the step and a tile of output columns (64 gate
+// and the 64 matching up columns, or 128 columns of down).  It lists the rows of its 256 that chose the expert, in row
+// order, and walks them 64 at a time: wave w multiplies rows 16 w .. 16 w + 15 of the 64 by the whole column tile
+// with `v_mfma_f32_16x16x32_bf16`.  The weight tile of a k step (128 rows of 32) goes through LDS once for the four
+// waves; a wave's own rows come straight from memory, sixteen bytes a lane, which is the A operand as it lies.  The
+// next k step's loads are in flight while this one's products run.  K a multiple of 8; rows 16-byte aligned.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kMoeChunk = 256;     // rows of the step a workgroup looks through
+constexpr int kMoeCols = 128;      // weight rows of a tile (gate|up: 64 + 64)
+constexpr int kMoeLdsRow = 40;     // bfloat16 a weight row of 32 takes in LDS (80 bytes: no two lanes of a read on one bank)
+
+template <bool GATE_UP>
+__global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __restrict__ x, long long x_stride,
+                                                              const bf16* __restrict__ w, const int* __restrict__ ids,
+                                                              void* __restrict__ out, int tokens, int top, int N, int K) {
+  __shared__ int list_src[kMoeChunk], list_dst[kMoeChunk];
+  __shared__ int wave_count[4];
+  __shared__ __attribute__((aligned(16))) bf16 wt[kMoeCols * kMoeLdsRow];
+  const int e = blockIdx.z;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n = lane % 16, g = lane / 16;
+  {
+    const int t = blockIdx.x * kMoeChunk + threadIdx.x;
+    int slot = -1;
+    if (t < tokens)
+      for (int k = 0; k < top; ++k)
+        if (ids[static_cast<int64_t>(t) * top + k] == e) slot = k;
+    const unsigned long long chose = __ballot(slot >= 0);
+    if (lane == 0) wave_count[wave] = __popcll(chose);
+    __syncthreads();
+    int before = 0;
+    for (int i = 0; i < wave; ++i) before += wave_count[i];
+    if (slot >= 0) {
+      const int rank = before + __popcll(chose & ((1ull << lane) - 1ull));
+      list_src[rank] = GATE_UP ? t : t * top + slot;
+      list_dst[rank] = t * top + slot;
+    }
+    __syncthreads();
+  }
+  const int rows = wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
+  if (rows == 0) return;
+  const int cols = GATE_UP ? kMoeCols / 2 : kMoeCols;     // output columns of the tile
+  const int n0 = blockIdx.y * cols;
+  const bf16* we = w + static_cast<int64_t>(e) * (GATE_UP ? 2 : 1) * N * K;
+  // the weight row this thread copies into LDS (two pieces of 8 of a row of 32), or none past N
+  const int wr = threadIdx.x / 2, wpiece = (threadIdx.x % 2) * 16;
+  const int wcol = GATE_UP ? (wr < 64 ? n0 + wr : n0 + wr - 64) : n0 + wr;
+  const bool w_in = wcol < N;
+  const bf16* wsrc = we + static_cast<int64_t>(GATE_UP && wr >= 64 ? N + wcol : wcol) * K;
+  const u32x4_t zero = {0, 0, 0, 0};
+  for (int sub = 0; sub * 64 < rows; ++sub) {
+    const int r = sub * 64 + wave * 16 + n;
+    const bf16* arow = x + static_cast<int64_t>(list_src[min(r, rows - 1)]) * x_stride;
+    f32x4_t acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    u32x4_t a_next, w_next[2];
+    auto fetch = [&](int k0) {
+      const int ka = k0 + 8 * g;
+      a_next = ka < K ? *reinterpret_cast<const u32x4_t*>(arow + ka) : zero;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int kw = k0 + wpiece + 8 * h;
+        w_next[h] = (w_in && kw < K) ? *reinterpret_cast<const u32x4_t*>(wsrc + kw) : zero;
+      }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += 32) {
+      const u32x4_t a_now = a_next;
+      __syncthreads();      // the tile before has been read by every wave
+#pragma unroll
+      for (int h = 0; h < 2; ++h) *reinterpret_cast<u32x4_t*>(&wt[wr * kMoeLdsRow + wpiece + 8 * h]) = w_next[h];
+      __syncthreads();
+      if (k0 + 32 < K) fetch(k0 + 32);
+      const bf16x8_t a_op = __builtin_bit_cast(bf16x8_t, a_now);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const u32x4_t b = *reinterpret_cast<const u32x4_t*>(&wt[(16 * j + n) * kMoeLdsRow + 8 * g]);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op, __builtin_bit_cast(bf16x8_t, b), acc[j], 0, 0, 0);
+      }
+    }
+    // acc[j][i] is the product of row 4 g + i of the wave's sixteen and weight row 16 j + n of the tile
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int rr = sub * 64 + wave * 16 + 4 * g + i;
+      if (rr >= rows) continue;
+      const int64_t dst = static_cast<int64_t>(list_dst[rr]) * N;
+      if (GATE_UP) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int col = n0 + 16 * j + n;
+          const float gt = acc[j][i];
+          if (col < N) static_cast<bf16*>(out)[dst + col] = from_float<bf16>(gt / (1.0f + expf(-gt)) * acc[j + 4][i]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int col = n0 + 16 * j + n;
+          if (col < N) static_cast<float*>(out)[dst + col] = acc[j][i];
+        }
+      }
+    }
+    __syncthreads();        // before the next 64 rows overwrite the tile
+  }
+}
+
 }  // namespace arle
 
 using namespace arle;
@@ -229,8 +338,18 @@ extern "C" int arle_moe_expert(const void* x, long long x_stride, const void* w,
   if (tokens == 0) return 0;
   if (experts < 1 || experts > 65535 || top < 1 || N < 1 || K < 1 || (N + kEN - 1) / kEN > 65535)
     return static_cast<int>(hipErrorInvalidValue);
-  const dim3 grid((tokens + kEM - 1) / kEM, (N + kEN - 1) / kEN, experts);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == kBF16 && K % 8 == 0 && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+    const int cols = gate_up ? kMoeCols / 2 : kMoeCols;
+    const dim3 mgrid((tokens + kMoeChunk - 1) / kMoeChunk, (N + cols - 1) / cols, experts);
+    if (gate_up)
+      moe_expert_mfma_kernel<true><<<mgrid, 256, 0, s>>>(static_cast<const bf16*>(x), x_stride, static_cast<const bf16*>(w), ids, out, tokens, top, N, K);
+    else
+      moe_expert_mfma_kernel<false><<<mgrid, 256, 0, s>>>(static_cast<const bf16*>(x), x_stride, static_cast<const bf16*>(w), ids, out, tokens, top, N, K);
+    return launch_status();
+  }
+  const dim3 grid((tokens + kEM - 1) / kEM, (N + kEN - 1) / kEN, experts);
 #define ARLE_EXPERT(TT, GU)                                                                                         \
   moe_expert_kernel<TT, GU><<<grid, kExpertThreads, 0, s>>>(static_cast<const TT*>(x), x_stride,                    \
                                                             static_cast<const TT*>(w), ids, out, tokens, top, N, K)

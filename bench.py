@@ -4,6 +4,7 @@
     python bench.py --workload qwen3-8b-mixed | qwen3-32b-decode     (two further workloads)
     python bench.py --generate                                       (the decode workload through LLM.generate)
     python bench.py --workload gufasun [--shape 4b|8b] [--layers L]  (the Gufasun design beside Qwen3 at equal sizes)
+    python bench.py --workload sovutar [--shape 4b|8b] [--layers L]  (the Sovutar design beside Qwen3 at equal sizes)
 
 A step is one decode step of `batch` requests, each holding a `prompt`-token random prompt
 (prefilled by the engine itself before the clock starts) and growing by one token per step.
@@ -782,20 +783,88 @@ def qwen3_work(q: dict, layers: int, tokens: int, batch: int, context: int) -> d
             "attn_mfma_kernel": attn, "attn_prefill_dma_kernel": attn, "attn_prefill_lds_kernel": attn}
 
 
-def gufasun_bench(args) -> int:
-    """Prefill and decode throughput of the Gufasun design and of Qwen3 at the same widths and depth, one JSON line
-    each, and the time of a step by kernel family with what each new kernel reaches of its roofline."""
-    import torch
+# ---- the Sovutar design beside Qwen3 at equal sizes -------------------------------------------------------
+# The widths and head counts of Qwen3-4B / 8B; layers alternate between the chunked attention (values mixed with the
+# first layer's) and the latent attention (a latent of 192 and a rotated part of 64: keys of 256, the widest the
+# matrix-core attention takes); sixteen experts of which four are chosen, and a shared one.
+SOVUTAR_SHAPES = {"4b": (QWEN3_4B, 1024, 1536), "8b": (QWEN3_8B, 2048, 2048)}      # (widths, window and chunk, expert size)
 
+
+def sovutar_config(shape: str, layers: int) -> dict:
+    q, span, ff = SOVUTAR_SHAPES[shape]
+    H, D = q["num_attention_heads"], q["head_dim"]
+    attn = {"heads": H, "kv_heads": q["num_key_value_heads"], "dim": D, "vdim": D, "scale": D ** -0.5,
+            "mask": {"size": span}, "v_mix": True}
+    lat = {"heads": H, "dim": D, "rot_dim": 64, "vdim": D, "kv_rank": 192, "scale": (D + 64) ** -0.5,
+           "mask": {"size": span}, "rot": {"base": 1000000.0, "dims": 64}}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": 16, "top": 4, "scale": 2.5}, "shared": {"ff": ff}}
+    out = [{"type": "attention", "mixer": dict(attn), "mlp": dict(mlp)} if i % 2 == 0 else
+           {"type": "latent_attention", "mixer": dict(lat), "mlp": dict(mlp)} for i in range(layers)]
+    return {"architecture": "Sovutar", "vocab": q["vocab_size"], "width": q["hidden_size"], "norm": {"eps": 1e-6},
+            "logit_softcap": 30.0, "layers": out}
+
+
+def sovutar_work(raw: dict, q: dict, tokens: int, batch: int, context: int) -> dict:
+    """Ideal work of the kernels that are new with this design, per step: kernel family -> (bytes, flops)."""
+    W, L = raw["width"], len(raw["layers"])
+    a = next(l["mixer"] for l in raw["layers"] if l["type"] == "attention")
+    m = next(l["mixer"] for l in raw["layers"] if l["type"] == "latent_attention")
+    n_att = sum(l["type"] == "attention" for l in raw["layers"])
+    n_lat = L - n_att
+    mlp = raw["layers"][0]["mlp"]
+    E, top, F = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"]
+    H, G, D, Dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+    LH, LD, R, LDv, C = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+    decode = tokens == batch
+    span = a["mask"]["size"]
+    keys_a = (context % span if decode else min(span, tokens) / 2) or 1
+    keys_l = min(m["mask"]["size"], context) if decode else min(m["mask"]["size"], tokens / 2)
+    attn_bytes = (n_att * batch * keys_a * G * (D + Dv) * 2 + n_lat * batch * keys_l * (2 * C + R) * 2) if decode else 0
+    attn_flops = n_att * tokens * keys_a * H * 2 * (D + Dv) + n_lat * tokens * keys_l * LH * 2 * (2 * C + R)
+    active = min(E, batch * top) if decode else E
+    return {
+        "norm_add_kernel": (tokens * W * (L * (4 + 8 + 2) + L * ((top + 1) * 4 + 8 + 2)), 0),
+        "wide_norm_store_kernel": (n_att * tokens * (H * D + G * D + G * Dv) * 4, 0),
+        "latent_prep_kernel": (n_lat * tokens * (LH * R * 2 + (C + R) + 2 * C + R) * 2, 0),
+        "head_proj": (n_lat * (tokens * LH * (LD + 2 * C + LDv) * 2 + LH * C * (LD + LDv) * 2),
+                      n_lat * tokens * LH * C * (LD + LDv) * 2),
+        "attn_softcap_mfma_kernel": (attn_bytes, attn_flops),
+        "moe_route_kernel": (L * (tokens + E) * W * 2, 0),
+        "moe_expert": (L * (active * 3 * W * F * 2 + tokens * top * (W * 2 + F * 4 + W * 4)), L * tokens * top * 3 * W * F * 2),
+    }
+
+
+def sovutar_bench(args) -> int:
+    """Prefill and decode throughput of the Sovutar design and of Qwen3 at the same widths and depth."""
+    from arle_amd.config import Qwen3Config, SovutarConfig
+
+    layers = args.layers if args.layers != FULL_LAYERS else 8
+    q = dict(SOVUTAR_SHAPES[args.shape][0], num_hidden_layers=layers)
+    raw = sovutar_config(args.shape, layers)
+    models = {"sovutar": ("Sovutar", SovutarConfig.from_dict(raw)), "qwen3": ("Qwen3ForCausalLM", Qwen3Config.from_dict(q))}
+    return design_bench(args, "sovutar", models, q, layers, lambda tokens, batch, context: sovutar_work(raw, q, tokens, batch, context))
+
+
+def gufasun_bench(args) -> int:
+    """Prefill and decode throughput of the Gufasun design and of Qwen3 at the same widths and depth."""
     from arle_amd.config import GufasunConfig, Qwen3Config
-    from arle_amd.engine import Engine, StepEntry
-    from arle_amd.kernels import ops
 
     layers = args.layers if args.layers != FULL_LAYERS else 8
     q = dict(GUFASUN_SHAPES[args.shape][0], num_hidden_layers=layers)
     raw = gufasun_config(args.shape, layers)
-    batch, prompt = args.batch or 8, args.prompt_len
     models = {"gufasun": ("Gufasun", GufasunConfig.from_dict(raw)), "qwen3": ("Qwen3ForCausalLM", Qwen3Config.from_dict(q))}
+    return design_bench(args, "gufasun", models, q, layers, lambda tokens, batch, context: gufasun_work(raw, q, tokens, batch, context))
+
+
+def design_bench(args, design: str, models: dict, q: dict, layers: int, design_work) -> int:
+    """Prefill and decode throughput of a design and of Qwen3 at the same widths and depth, one JSON line each, and the
+    time of a step by kernel family with what each new kernel reaches of its roofline."""
+    import torch
+
+    from arle_amd.engine import Engine, StepEntry
+    from arle_amd.kernels import ops
+
+    batch, prompt = args.batch or 8, args.prompt_len
     gen = torch.Generator().manual_seed(1234)
     toks = lambda n: torch.randint(0, q["vocab_size"], (n,), generator=gen).tolist()
     lines = []
@@ -845,8 +914,8 @@ def gufasun_bench(args) -> int:
             t = toks(prompt)
             pre, dec = profiled_steps(torch, [lambda: engine.step([StepEntry("prof", t, [prompt - 1])]), decode_step])
             engine.end_request("prof")
-            work = {"prefill": gufasun_work(raw, q, prompt, 1, 0) if name == "gufasun" else qwen3_work(q, layers, prompt, 1, 0),
-                    "decode": gufasun_work(raw, q, batch, batch, prompt) if name == "gufasun" else qwen3_work(q, layers, batch, batch, prompt)}
+            work = {"prefill": design_work(prompt, 1, 0) if name == design else qwen3_work(q, layers, prompt, 1, 0),
+                    "decode": design_work(batch, batch, prompt) if name == design else qwen3_work(q, layers, batch, batch, prompt)}
             for phase, step in (("prefill", pre), ("decode", dec)):
                 fam: dict = {}
                 for kname, us in step:
@@ -912,10 +981,10 @@ def main() -> int:
                          "and write the table that ARLE_AMD_PRODUCT_TABLE / ops.load_product_table reads; WIDTHS: 4b, 8b, "
                          "32b or hidden,q_width,kv_width,intermediate[,vocabulary]")
     ap.add_argument("--out", default=None, help="--tune-products: the table's file (default: product_table_<widths>.json)")
-    ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode", "gufasun"],
+    ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode", "gufasun", "sovutar"],
                     help="qwen3-4b is the default run; the next two are further workloads at larger shapes; gufasun: "
                          "the Gufasun design beside Qwen3 at equal widths and depth (--shape, --layers, --batch, --prompt-len)")
-    ap.add_argument("--shape", default="4b", choices=["4b", "8b"], help="--workload gufasun: whose widths")
+    ap.add_argument("--shape", default="4b", choices=["4b", "8b"], help="--workload gufasun / sovutar: whose widths")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
@@ -937,6 +1006,8 @@ def main() -> int:
         return step_gaps(args)
     if args.workload == "gufasun":
         return gufasun_bench(args)
+    if args.workload == "sovutar":
+        return sovutar_bench(args)
     if args.workload == "qwen3-4b" and args.batch is None:
         args.batch = 8
     if args.workload != "qwen3-4b":
