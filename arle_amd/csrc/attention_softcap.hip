@@ -361,11 +361,13 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
   int seg, row, head, kvh, first_row, last_row;
   bool live;
   if (HEADS) {
+    // a kv head with more than sixteen q heads is taken by several workgroups, sixteen q heads each
+    const int parts = (group + 15) / 16, part = blockIdx.y % parts;
     seg = blockIdx.x;
-    kvh = blockIdx.y;
+    kvh = blockIdx.y / parts;
     row = first_row = last_row = a.seg_row0[seg];
-    head = kvh * group + min(n, group - 1);
-    live = n < group;
+    head = kvh * group + min(16 * part + n, group - 1);
+    live = 16 * part + n < group;
   } else {
     // the blockIdx.x-th block of sixteen rows, counted through the segments
     int left = blockIdx.x, found = -1;
@@ -600,11 +602,29 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
 }
 
 constexpr int kCapSplitWaves = 8;   // waves that share the keys of a decoded row
+constexpr int kCapLdsMost = 160 * 1024;   // LDS of a gfx950 compute unit: no workgroup can ask for more
+
+// What a workgroup may ask for on this device (never more than kCapLdsMost), asked once.
+inline int cap_lds_limit() {
+  static int limit = 0;
+  if (limit == 0) {
+    int dev = 0, value = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&value, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && value > 0)
+      limit = value < kCapLdsMost ? value : kCapLdsMost;
+    else
+      limit = 64 * 1024;
+  }
+  return limit;
+}
 
 }  // namespace arle
 
+// Bytes of LDS that a workgroup of the matrix-core kernel may use on this device (the return value, not an error code).
+extern "C" int arle_attn_softcap_lds_limit() { return cap_lds_limit(); }
+
 // bfloat16 only.  Dk a multiple of 8 up to 256, Dv a multiple of 16 up to 256, page_size a multiple of 16, rows of
-// q and out 16-byte aligned (strides multiples of 8).  heads_mode: every segment is one row and nq / nkv <= 16.
+// q and out 16-byte aligned (strides multiples of 8).  heads_mode: every segment is one row.
 // row_blocks: an upper bound of the sixteen-row blocks of all segments (blocks past the last one return).
 extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* out, long long o_stride,
                                       const void* k_pages, const void* v_pages, const int* block_table,
@@ -615,7 +635,7 @@ extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* o
                                       void* stream) {
   if (segments == 0) return 0;
   if (Dk % 8 || Dk > 256 || Dv % 16 || Dv > 256 || page_size % 16 || nkv < 1 || nq % nkv || nq > 65535 ||
-      (heads_mode && nq / nkv > 16) || window < 0 || chunk < 0)
+      window < 0 || chunk < 0)
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const CapArgs a{static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), o_stride,
@@ -633,19 +653,21 @@ extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* o
   const int group = nq / nkv;
   const int head_waves = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);   // q heads of one kv head that share a workgroup
   const size_t merge_bytes = static_cast<size_t>(kCapSplitWaves) * ((Dv / 16) * kWave * 4 + 32) * sizeof(float) + page_bytes;
+  if (heads_mode && merge_bytes > static_cast<size_t>(cap_lds_limit())) return static_cast<int>(hipErrorInvalidValue);
 #define ARLE_CAP(KC, VC)                                                                                           \
   do {                                                                                                             \
     if (heads_mode) {                                                                                              \
       static bool raised = false;   /* more LDS than a launch gets unasked: said once for the kernel */            \
       if (!raised && merge_bytes > 48 * 1024) {                                                                    \
+        const int most = kCapSplitWaves * (VC * kWave * 4 + 32) * 4 + 48 * 1024;                                   \
         const hipError_t e = hipFuncSetAttribute(                                                                  \
             reinterpret_cast<const void*>(&attn_softcap_mfma_kernel<KC, VC, true, kCapSplitWaves>),                \
-            hipFuncAttributeMaxDynamicSharedMemorySize, kCapSplitWaves * (VC * kWave * 4 + 32) * 4 + 48 * 1024);              \
+            hipFuncAttributeMaxDynamicSharedMemorySize, most < cap_lds_limit() ? most : cap_lds_limit());              \
         if (e != hipSuccess) return static_cast<int>(e);                                                           \
         raised = true;                                                                                             \
       }                                                                                                            \
       attn_softcap_mfma_kernel<KC, VC, true, kCapSplitWaves>                                                       \
-          <<<dim3(segments, nkv), kCapSplitWaves * kWave, merge_bytes, s>>>(a);                                    \
+          <<<dim3(segments, nkv * ((group + 15) / 16)), kCapSplitWaves * kWave, merge_bytes, s>>>(a);                                    \
     }                                                                                                              \
     else if (head_waves == 4)                                                                                      \
       attn_softcap_mfma_kernel<KC, VC, false, 4><<<dim3(row_blocks, nq / 4), 4 * kWave, page_bytes, s>>>(a);                \

@@ -107,9 +107,74 @@ __global__ __launch_bounds__(kProjThreads) void head_proj_kernel(const T* __rest
       out[static_cast<int64_t>(row0 + r) * out_stride + static_cast<int64_t>(h) * out_head + n] = from_float<T>(acc[r]);
 }
 
+// ---- matrix-core form (bfloat16) -----------------------------------------------------------------
+// The same product with every head's matrix stored [N, K] (K-major), so that both operands of
+// `v_mfma_f32_16x16x32_bf16` are sixteen consecutive bytes a lane, straight from memory: a head's matrix is a few
+// dozen kilobytes and stays in the caches.  A wave takes sixteen rows and sixty-four columns of one head; the four
+// waves of a workgroup take sixty-four rows.  K a multiple of 8, heads' offsets multiples of 8, rows 16-byte aligned.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void head_proj_mfma_kernel(const bf16* __restrict__ in, long long in_stride, int in_head,
+                                                             const bf16* __restrict__ wnk, bf16* __restrict__ out,
+                                                             long long out_stride, int out_head, int rows, int K, int N) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n = lane % 16, g = lane / 16;
+  const int h = blockIdx.y, n0 = blockIdx.z * 64;
+  const int row0 = blockIdx.x * 64 + wave * 16;
+  if (row0 >= rows) return;
+  const bf16* arow = in + static_cast<int64_t>(min(row0 + n, rows - 1)) * in_stride + static_cast<int64_t>(h) * in_head;
+  const bf16* wh = wnk + static_cast<int64_t>(h) * N * K;
+  const bf16* wrow[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) wrow[j] = wh + static_cast<int64_t>(min(n0 + 16 * j + n, N - 1)) * K;
+  f32x4_t acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const u32x4_t zero = {0, 0, 0, 0};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const int k = min(k0 + 8 * g, K - 8);      // a piece past K is the last piece again, and zeroed
+    const bool in_k = k0 + 8 * g < K;
+    const u32x4_t a_raw = *reinterpret_cast<const u32x4_t*>(arow + k);
+    u32x4_t b_raw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b_raw[j] = *reinterpret_cast<const u32x4_t*>(wrow[j] + k);
+    const bf16x8_t a_op = __builtin_bit_cast(bf16x8_t, in_k ? a_raw : zero);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op, __builtin_bit_cast(bf16x8_t, b_raw[j]), acc[j], 0, 0, 0);
+  }
+  // acc[j][i]: row 4 g + i of the wave's sixteen, column 16 j + n of the tile
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = row0 + 4 * g + i;
+    if (r >= rows) continue;
+    bf16* orow = out + static_cast<int64_t>(r) * out_stride + static_cast<int64_t>(h) * out_head;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = n0 + 16 * j + n;
+      if (col < N) orow[col] = from_float<bf16>(acc[j][i]);
+    }
+  }
+}
+
 }  // namespace arle
 
 using namespace arle;
+
+// bfloat16; wnk [heads, N, K].
+extern "C" int arle_head_proj_mfma(const void* in, long long in_stride, int in_head, const void* wnk, void* out,
+                                   long long out_stride, int out_head, int rows, int heads, int K, int N, void* stream) {
+  if (rows == 0) return 0;
+  if (heads < 1 || heads > 65535 || K < 8 || K % 8 || in_head % 8 || in_stride % 8 || N < 1 || (N + 63) / 64 > 65535 ||
+      reinterpret_cast<uintptr_t>(in) % 16 || reinterpret_cast<uintptr_t>(wnk) % 16)
+    return static_cast<int>(hipErrorInvalidValue);
+  const dim3 grid((rows + 63) / 64, heads, (N + 63) / 64);
+  head_proj_mfma_kernel<<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const bf16*>(in), in_stride, in_head, static_cast<const bf16*>(wnk), static_cast<bf16*>(out), out_stride,
+      out_head, rows, K, N);
+  return launch_status();
+}
 
 // q [T, heads*(D+R)], dkv [T, C+R] and q_full [T, heads*(C+R)] of `dtype`, as the pages: k_pages
 // [pages, 1, page_size, C+R], v_pages [pages, 1, C, page_size].  cos, sin: float32 [positions, rot/2].

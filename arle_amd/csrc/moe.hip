@@ -4,7 +4,7 @@
 //   lower index);  weight of a chosen expert = s / (sum of the chosen s + 1e-20) * scale.
 //   expert e: down_e (silu(gate_e h) * (up_e h)).
 //
-// `moe_route`: one wave a token.  `moe_expert`: a workgroup takes one expert, 64 consecutive rows of the step and 64
+// `moe_route`: one workgroup a token.  `moe_expert`: a workgroup takes one expert, 64 consecutive rows of the step and 64
 // output columns; it lists the rows of its 64 that chose the expert (in row order) and multiplies only those, so no
 // step sorts anything and a launch's shape follows the number of rows alone.  The result of (token t, its k-th
 // choice) lies at row t * top + k: the gate|up pass leaves the activation there, the down pass the expert's output,
@@ -34,33 +34,47 @@ __device__ __forceinline__ Best wave_best(Best b) {
   return b;
 }
 
-template <typename T, typename TW>
-__global__ __launch_bounds__(kWave) void moe_route_kernel(const T* __restrict__ x, long long x_stride,
-                                                          const TW* __restrict__ w, const void* __restrict__ correction,
-                                                          int c_dtype, int* __restrict__ ids, float* __restrict__ weights,
-                                                          int width, int experts, int top, float scale) {
+constexpr int kRouteThreads = 256;
+
+// One workgroup a token: the row goes to LDS as floats once; wave w computes the logits of experts w, w + 4, ...
+// (eight consecutive entries a lane and step where the width allows, one otherwise: an order that depends on the
+// width alone); then the first wave picks the `top` experts one after the other.
+template <typename T, typename TW, bool VEC>
+__global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __restrict__ x, long long x_stride,
+                                                                  const TW* __restrict__ w, const void* __restrict__ correction,
+                                                                  int c_dtype, int* __restrict__ ids, float* __restrict__ weights,
+                                                                  int width, int experts, int top, float scale) {
+  extern __shared__ float route_lds[];   // [width] the row, then [experts] the scores
+  float* xs = route_lds;
+  float* score = route_lds + width;
   const int64_t t = blockIdx.x;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const T* row = x + t * x_stride;
+  for (int i = threadIdx.x; i < width; i += kRouteThreads) xs[i] = to_float(row[i]);
+  __syncthreads();
+  for (int e = wave; e < experts; e += kRouteThreads / kWave) {
+    const TW* we = w + static_cast<int64_t>(e) * width;
+    float dot = 0.f;
+    if (VEC) {
+      for (int i = 8 * lane; i < width; i += 8 * kWave) {
+        const float4 lo = ld4<TW>(we + i), hi = ld4<TW>(we + i + 4);
+        dot = fmaf(xs[i], lo.x, dot); dot = fmaf(xs[i + 1], lo.y, dot); dot = fmaf(xs[i + 2], lo.z, dot); dot = fmaf(xs[i + 3], lo.w, dot);
+        dot = fmaf(xs[i + 4], hi.x, dot); dot = fmaf(xs[i + 5], hi.y, dot); dot = fmaf(xs[i + 6], hi.z, dot); dot = fmaf(xs[i + 7], hi.w, dot);
+      }
+    } else {
+      for (int i = lane; i < width; i += kWave) dot = fmaf(xs[i], to_float(we[i]), dot);
+    }
+    dot = wave_sum(dot);
+    if (lane == 0) score[e] = 1.0f / (1.0f + expf(-dot));
+  }
+  __syncthreads();
+  if (wave != 0) return;
   float s[kMaxExpertsPerLane], choice[kMaxExpertsPerLane];
 #pragma unroll
   for (int j = 0; j < kMaxExpertsPerLane; ++j) {
-    s[j] = 0.f;
-    choice[j] = -INFINITY;
-  }
-  for (int e = 0; e < experts; ++e) {
-    const TW* we = w + static_cast<int64_t>(e) * width;
-    float dot = 0.f;
-    for (int i = lane; i < width; i += kWave) dot = fmaf(to_float(row[i]), to_float(we[i]), dot);
-    dot = wave_sum(dot);
-    const float sg = 1.0f / (1.0f + expf(-dot));
-#pragma unroll
-    for (int j = 0; j < kMaxExpertsPerLane; ++j) {
-      if (e == lane + j * kWave) {
-        s[j] = sg;
-        choice[j] = sg + (correction ? load_as_float(correction, c_dtype, e) : 0.f);
-      }
-    }
+    const int e = lane + j * kWave;
+    s[j] = e < experts ? score[e] : 0.f;
+    choice[j] = e < experts ? s[j] + (correction ? load_as_float(correction, c_dtype, e) : 0.f) : -INFINITY;
   }
   float sum = 0.f, mine = 0.f;   // lane k keeps the k-th chosen score (top <= 64)
   int mine_id = 0;
@@ -319,15 +333,34 @@ extern "C" int arle_moe_route(const void* x, long long x_stride, int x_dtype, co
   if (experts < 1 || experts > kWave * kMaxExpertsPerLane || top < 1 || top > experts || top > kWave)
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
-#define ARLE_ROUTE(TX, TWT)                                                                                       \
-  moe_route_kernel<TX, TWT><<<tokens, kWave, 0, s>>>(static_cast<const TX*>(x), x_stride, static_cast<const TWT*>(w), \
-                                                     correction, c_dtype, ids, weights, width, experts, top, scale)
+  const size_t lds = static_cast<size_t>(width + experts) * sizeof(float);
+  if (lds > 60 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  const bool vec = width % 8 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
+#define ARLE_ROUTE_V(TX, TWT, V)                                                                                   \
+  do {                                                                                                             \
+    static bool raised = false;                                                                                    \
+    if (!raised && lds > 48 * 1024) {                                                                              \
+      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_route_kernel<TX, TWT, V>),     \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 60 * 1024);           \
+      if (err != hipSuccess) return static_cast<int>(err);                                                         \
+      raised = true;                                                                                               \
+    }                                                                                                              \
+    moe_route_kernel<TX, TWT, V><<<tokens, kRouteThreads, lds, s>>>(static_cast<const TX*>(x), x_stride,           \
+                                                                    static_cast<const TWT*>(w), correction, c_dtype, \
+                                                                    ids, weights, width, experts, top, scale);      \
+  } while (0)
+#define ARLE_ROUTE(TX, TWT)                          \
+  do {                                               \
+    if (vec) ARLE_ROUTE_V(TX, TWT, true);            \
+    else ARLE_ROUTE_V(TX, TWT, false);               \
+  } while (0)
   if (x_dtype == kF32) {
     if (w_dtype == kF32) ARLE_ROUTE(float, float); else ARLE_ROUTE(float, bf16);
   } else {
     if (w_dtype == kF32) ARLE_ROUTE(bf16, float); else ARLE_ROUTE(bf16, bf16);
   }
 #undef ARLE_ROUTE
+#undef ARLE_ROUTE_V
   return launch_status();
 }
 

@@ -4,8 +4,8 @@
 //   res_j += y_j / sqrt(mean_j(y_j^2) + eps) * (w_j  or  1 + w_j)
 //   act_j = res_j rounded to the activation type  (what the next sublayer reads; optional)
 //
-// An addend is a tensor [T, W], or parts that are added in ascending order: the float32 partial products of a
-// matrix product whose K was split (part p of row t at p * part_stride + t * row_stride), or the outputs of the
+// An addend is a float32 tensor [T, W], or parts that are added in ascending order: the float32 partial products of
+// a matrix product whose K was split (part p of row t at p * part_stride + t * row_stride), or the outputs of the
 // experts that a token chose, [T, n, W] with a weight per (token, part).  The sums, the statistics, the weight and
 // the residual are 32-bit.  A row's arithmetic depends on nothing but the row.
 #include "common.h"
@@ -16,26 +16,41 @@ constexpr int kPostThreads = 256;
 constexpr int kPostWaves = kPostThreads / kWave;
 
 struct Addend {
-  const void* p;          // null: no addend
+  const float* p;         // null: no addend
   int parts;              // parts added in order (>= 1)
   long long part_stride;  // elements between parts of one row
   long long row_stride;   // elements between rows
-  int dtype;              // kF32 / kBF16
   const float* weights;   // [T, parts] factors, or null
 };
 
-__device__ __forceinline__ float addend_at(const Addend& a, int64_t row, int i) {
-  const int64_t base = row * a.row_stride + i;
-  float sum = load_as_float(a.p, a.dtype, base);
-  if (a.weights) sum *= a.weights[row * a.parts];
+// Four consecutive entries of an addend's row: its parts added in ascending order (weighted where it has weights).
+// Every load is typed and stands under no condition on data, so the parts' loads are in flight together.
+template <bool VEC>
+__device__ __forceinline__ float4 addend_at(const Addend& a, int64_t row, int i) {
+  const float* base = a.p + row * a.row_stride + i;
+  auto get = [&](int p) {
+    if (VEC) return *reinterpret_cast<const float4*>(base + p * a.part_stride);
+    return float4{base[p * a.part_stride], 0.f, 0.f, 0.f};
+  };
+  float4 sum = get(0);
+  if (a.weights) {
+    const float f = a.weights[row * a.parts];
+    sum.x *= f; sum.y *= f; sum.z *= f; sum.w *= f;
+  }
   for (int p = 1; p < a.parts; ++p) {
-    const float v = load_as_float(a.p, a.dtype, base + p * a.part_stride);
-    sum = a.weights ? fmaf(a.weights[row * a.parts + p], v, sum) : sum + v;
+    const float4 v = get(p);
+    if (a.weights) {
+      const float f = a.weights[row * a.parts + p];
+      sum.x = fmaf(f, v.x, sum.x); sum.y = fmaf(f, v.y, sum.y); sum.z = fmaf(f, v.z, sum.z); sum.w = fmaf(f, v.w, sum.w);
+    } else {
+      sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+    }
   }
   return sum;
 }
 
-template <typename TAct, typename TW>
+// VEC: width a multiple of 4 and every pointer and stride 16-byte aligned; a thread takes four entries at a time.
+template <typename TAct, typename TW, bool VEC>
 __global__ __launch_bounds__(kPostThreads) void norm_add_kernel(float* __restrict__ residual, const Addend a,
                                                                 const Addend b, const TW* __restrict__ w,
                                                                 int one_plus, TAct* __restrict__ act, int width,
@@ -43,21 +58,39 @@ __global__ __launch_bounds__(kPostThreads) void norm_add_kernel(float* __restric
   extern __shared__ float ys[];  // [width]
   __shared__ float lds[kPostWaves];
   const int64_t r = blockIdx.x;
+  constexpr int kStep = VEC ? 4 : 1;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += kPostThreads) {
-    float y = addend_at(a, r, i);
-    if (b.p) y += addend_at(b, r, i);
-    ys[i] = y;
-    ss = fmaf(y, y, ss);
+  for (int i = kStep * threadIdx.x; i < width; i += kStep * kPostThreads) {
+    float4 y = addend_at<VEC>(a, r, i);
+    if (b.p) {
+      const float4 z = addend_at<VEC>(b, r, i);
+      y.x += z.x; y.y += z.y; y.z += z.z; y.w += z.w;
+    }
+    if (VEC) {
+      *reinterpret_cast<float4*>(ys + i) = y;
+      ss = fmaf(y.x, y.x, ss); ss = fmaf(y.y, y.y, ss); ss = fmaf(y.z, y.z, ss); ss = fmaf(y.w, y.w, ss);
+    } else {
+      ys[i] = y.x;
+      ss = fmaf(y.x, y.x, ss);
+    }
   }
   const float total = block_sum<kPostWaves>(ss, lds);
   const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
   float* res = residual + r * width;
-  for (int i = threadIdx.x; i < width; i += kPostThreads) {
-    const float g = one_plus ? 1.0f + to_float(w[i]) : to_float(w[i]);
-    const float v = res[i] + ys[i] * inv * g;
-    res[i] = v;
-    if (act) act[r * width + i] = from_float<TAct>(v);
+  const float one = one_plus ? 1.0f : 0.0f;
+  for (int i = kStep * threadIdx.x; i < width; i += kStep * kPostThreads) {
+    if (VEC) {
+      const float4 g = ld4<TW>(w + i), y = *reinterpret_cast<const float4*>(ys + i);
+      float4 v = *reinterpret_cast<const float4*>(res + i);
+      v.x = fmaf(y.x * inv, one + g.x, v.x); v.y = fmaf(y.y * inv, one + g.y, v.y);
+      v.z = fmaf(y.z * inv, one + g.z, v.z); v.w = fmaf(y.w * inv, one + g.w, v.w);
+      *reinterpret_cast<float4*>(res + i) = v;
+      if (act) st4<TAct>(act + r * width + i, v);
+    } else {
+      const float v = fmaf(ys[i] * inv, one + to_float(w[i]), res[i]);
+      res[i] = v;
+      if (act) act[r * width + i] = from_float<TAct>(v);
+    }
   }
 }
 
@@ -65,29 +98,37 @@ __global__ __launch_bounds__(kPostThreads) void norm_add_kernel(float* __restric
 
 using namespace arle;
 
-// residual float32 [rows, width], updated in place.  act: [rows, width] of act_dtype, or null.
-extern "C" int arle_norm_add(float* residual, const void* a, int a_parts, long long a_part_stride,
-                             long long a_row_stride, int a_dtype, const float* a_weights, const void* b, int b_parts,
-                             long long b_part_stride, long long b_row_stride, int b_dtype, const float* b_weights,
+// residual float32 [rows, width], updated in place.  Addends are float32.  act: [rows, width] of act_dtype, or null.
+extern "C" int arle_norm_add(float* residual, const float* a, int a_parts, long long a_part_stride,
+                             long long a_row_stride, const float* a_weights, const float* b, int b_parts,
+                             long long b_part_stride, long long b_row_stride, const float* b_weights,
                              const void* w, int w_dtype, int one_plus, void* act, int act_dtype, int rows, int width,
                              float eps, void* stream) {
   if (rows == 0) return 0;
   if (!a || a_parts < 1 || (b && b_parts < 1) || width < 1 || width > 16384) return static_cast<int>(hipErrorInvalidValue);
-  const Addend A{a, a_parts, a_part_stride, a_row_stride, a_dtype, a_weights};
-  const Addend B{b, b_parts, b_part_stride, b_row_stride, b_dtype, b_weights};
+  const Addend A{a, a_parts, a_part_stride, a_row_stride, a_weights};
+  const Addend B{b, b_parts, b_part_stride, b_row_stride, b_weights};
   hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t lds = static_cast<size_t>(width) * sizeof(float);
-#define ARLE_POST(TA, TWT)                                                                                     \
+  auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = width % 4 == 0 && al(residual) && al(a) && a_part_stride % 4 == 0 && a_row_stride % 4 == 0 &&
+                   (!b || (al(b) && b_part_stride % 4 == 0 && b_row_stride % 4 == 0)) && al(w) && al(act);
+#define ARLE_POST_V(TA, TWT, V)                                                                                \
   do {                                                                                                         \
     static bool raised = false;                                                                                \
     if (!raised && lds > 48 * 1024) {                                                                          \
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&norm_add_kernel<TA, TWT>),       \
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&norm_add_kernel<TA, TWT, V>),    \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);         \
       if (e != hipSuccess) return static_cast<int>(e);                                                         \
       raised = true;                                                                                           \
     }                                                                                                          \
-    norm_add_kernel<TA, TWT><<<rows, kPostThreads, lds, s>>>(residual, A, B, static_cast<const TWT*>(w), one_plus, \
-                                                             static_cast<TA*>(act), width, eps);               \
+    norm_add_kernel<TA, TWT, V><<<rows, kPostThreads, lds, s>>>(residual, A, B, static_cast<const TWT*>(w),    \
+                                                                one_plus, static_cast<TA*>(act), width, eps);  \
+  } while (0)
+#define ARLE_POST(TA, TWT)                     \
+  do {                                         \
+    if (vec) ARLE_POST_V(TA, TWT, true);       \
+    else ARLE_POST_V(TA, TWT, false);          \
   } while (0)
   if (act_dtype == kF32) {
     if (w_dtype == kF32) ARLE_POST(float, float); else ARLE_POST(float, bf16);
@@ -95,5 +136,6 @@ extern "C" int arle_norm_add(float* residual, const void* a, int a_parts, long l
     if (w_dtype == kF32) ARLE_POST(bf16, float); else ARLE_POST(bf16, bf16);
   }
 #undef ARLE_POST
+#undef ARLE_POST_V
   return launch_status();
 }

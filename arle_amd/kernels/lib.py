@@ -71,14 +71,15 @@ SIGNATURES = {
                                                      _f, _f, _p, _p, _i, _i, _i, _p, _i, _p]),
     "arle_attn_softcap_mfma": ("attention_softcap", [_p, _ll, _p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i,
                                                      _i, _f, _f, _p, _p, _i, _i, _i, _p, _i, _p]),
+    "arle_attn_softcap_lds_limit": ("attention_softcap", []),
     "arle_wide_norm_store": ("attention_softcap", [_p, _ll, _p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _p, _i, _f, _p, _p,
                                                    _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "arle_tanh_cap": ("elementwise", [_p, _ll, _f, _p]),
-    "arle_norm_add": ("post_norm", [_p, _p, _i, _ll, _ll, _i, _p, _p, _i, _ll, _ll, _i, _p, _p, _i, _i, _p, _i, _i, _i,
-                                    _f, _p]),
+    "arle_norm_add": ("post_norm", [_p, _p, _i, _ll, _ll, _p, _p, _i, _ll, _ll, _p, _p, _i, _i, _p, _i, _i, _i, _f, _p]),
     "arle_latent_prep": ("latent", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _i, _f, _p, _p, _i, _p, _p, _p, _i, _p, _p, _i, _i,
                                     _i, _i, _i, _i, _p]),
     "arle_head_proj": ("latent", [_p, _ll, _i, _p, _p, _ll, _i, _i, _i, _i, _i, _i, _p]),
+    "arle_head_proj_mfma": ("latent", [_p, _ll, _i, _p, _p, _ll, _i, _i, _i, _i, _i, _p]),
     "arle_moe_route": ("moe", [_p, _ll, _i, _p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _f, _p]),
     "arle_moe_expert": ("moe", [_p, _ll, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
     "arle_ceiling_read": ("ceilings", [_p, _ll, _i, _p, _p, _p]),

@@ -1674,11 +1674,16 @@ def attn_softcap_mfma_fits(window: int, table_width: int, page_size: int) -> boo
     return (seen // page_size + 2) * 4 <= 48 * 1024
 
 
+@functools.lru_cache(maxsize=None)
+def _softcap_lds_limit() -> int:
+    return int(lib.function("arle_attn_softcap_lds_limit")())
+
+
 def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *, max_qlen: int,
                       num_q_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
                       softcap: float = 0.0, r1=None, r2=None, window: int = 0, chunk: int = 0, sink=None):
     """`attn_softcap_simt` on the matrix cores, bfloat16: sixteen rows of a segment a wave, or (when every segment is
-    one decoded row and a kv head has at most sixteen q heads) one row's q heads of a kv head a wave."""
+    one decoded row) one row's q heads of a kv head, sixteen at a time, a wave."""
     _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, r1, r2, sink)
     _check_sink(sink, num_q_heads, window, chunk)
     tokens = q.shape[0]
@@ -1704,7 +1709,12 @@ def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot,
               and r1.is_contiguous() and r2.is_contiguous(), "r1, r2 must be [heads] of one type")
     _need(attn_softcap_mfma_fits(mask_span(window, chunk), block_table.shape[1], page_size),
           "the keys a row sees span more pages than the kernel holds ids for")
-    heads_mode = max_qlen == 1 and group <= 16 and segments == tokens
+    # a decoded row's waves add their sums through LDS: that and the page ids have to fit a compute unit's
+    mapped = block_table.shape[1] * page_size
+    span = mask_span(window, chunk)
+    page_ids = ((span + 16 if 0 < span and span + 16 < mapped else mapped) + 64) // page_size + 2
+    heads_mode = (max_qlen == 1 and segments == tokens
+                  and 8 * ((value_dim // 16) * 256 + 32) * 4 + page_ids * 4 <= _softcap_lds_limit())
     row_blocks = tokens // 16 + segments      # no fewer than the sixteen-row blocks of all segments together
     lib.call("arle_attn_softcap_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(),
              v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], seg_row0.data_ptr(), seg_slot.data_ptr(),
@@ -1757,21 +1767,21 @@ NORM_ADD_MAX_WIDTH = 16384
 
 
 def _addend_args(term, rows: int, width: int):
-    """(pointer, parts, part stride, row stride, type code, weights pointer) of one addend of `norm_add`: a tensor
-    [T, W]; a float32 stack [S, T, W] of partial sums; or (outputs [T, n, W], weights float32 [T, n])."""
+    """(pointer, parts, part stride, row stride, weights pointer) of one float32 addend of `norm_add`: a tensor [T, W];
+    a stack [S, T, W] of partial sums; or (outputs [T, n, W], weights [T, n])."""
     if term is None:
-        return (0, 0, 0, 0, 0, 0)
+        return (0, 0, 0, 0, 0)
     if isinstance(term, tuple):
         outs, weights = term
         _need(outs.dim() == 3 and outs.shape[0] == rows and outs.shape[2] == width and outs.is_contiguous()
-              and outs.dtype in _CODES, "weighted outputs must be contiguous [T, n, W]")
+              and outs.dtype == torch.float32, "weighted outputs must be contiguous float32 [T, n, W]")
         _need(weights.shape == outs.shape[:2] and weights.dtype == torch.float32 and weights.is_contiguous(),
               "their weights must be contiguous float32 [T, n]")
-        return (outs.data_ptr(), outs.shape[1], width, outs.shape[1] * width, _code(outs), weights.data_ptr())
-    _need(term.dim() in (2, 3) and tuple(term.shape[-2:]) == (rows, width) and term.is_contiguous() and term.dtype in _CODES,
-          "an addend must match the residual ([T, W] or a float32 stack [S, T, W])")
-    _need(term.dim() == 2 or (term.dtype == torch.float32 and term.shape[0] >= 1), "a stack of partial sums is float32")
-    return (term.data_ptr(), term.shape[0] if term.dim() == 3 else 1, rows * width, width, _code(term), 0)
+        return (outs.data_ptr(), outs.shape[1], width, outs.shape[1] * width, weights.data_ptr())
+    _need(term.dim() in (2, 3) and tuple(term.shape[-2:]) == (rows, width) and term.is_contiguous()
+          and term.dtype == torch.float32 and term.shape[0] >= 1,
+          "an addend must match the residual (float32 [T, W] or a stack [S, T, W])")
+    return (term.data_ptr(), term.shape[0] if term.dim() == 3 else 1, rows * width, width, 0)
 
 
 def norm_add(residual: torch.Tensor, terms, weight: torch.Tensor, eps: float, *, one_plus: bool = False,
@@ -1780,6 +1790,8 @@ def norm_add(residual: torch.Tensor, terms, weight: torch.Tensor, eps: float, *,
     returns the updated residual rounded to `act_dtype` (None: nothing is returned)."""
     terms = [t for t in (terms if isinstance(terms, list) else [terms]) if t is not None]
     _need(1 <= len(terms) <= 2, "norm_add takes one or two addends")
+    # what a sublayer leaves for the residual is 32-bit sums; an output that was rounded on its way is widened first
+    terms = [t.float() if torch.is_tensor(t) and t.dtype == torch.bfloat16 else t for t in terms]
     _gpu(residual, weight, *[x for t in terms for x in (t if isinstance(t, tuple) else (t,))])
     _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
           "residual must be contiguous float32 [T, W]")
@@ -1852,6 +1864,28 @@ def head_proj(x, wt, out, *, heads: int, in_head: int, out_head: int):
           and (heads - 1) * out_head + N <= out.shape[1], "a head's numbers must lie inside its row")
     lib.call("arle_head_proj", x.data_ptr(), x.stride(0), int(in_head), wt.data_ptr(), out.data_ptr(), out.stride(0),
              int(out_head), _code(x), x.shape[0], heads, K, N, _stream())
+    return out
+
+
+def head_proj_mfma_supported(x, heads: int, in_head: int, K: int) -> bool:
+    """Whether the matrix-core form of `head_proj` takes these operands (bfloat16, 16-byte pieces)."""
+    return (x.dtype == torch.bfloat16 and K % 8 == 0 and K >= 8 and in_head % 8 == 0 and x.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0)
+
+
+def head_proj_mfma(x, wnk, out, *, heads: int, in_head: int, out_head: int):
+    """`head_proj` on the matrix cores: bfloat16, every head's matrix stored wnk [heads, N, K]."""
+    _gpu(x, wnk, out)
+    _rows(x, "x")
+    _rows(out, "out")
+    _need(wnk.dim() == 3 and wnk.shape[0] == heads and wnk.is_contiguous(), "wnk must be contiguous [heads, N, K]")
+    N, K = wnk.shape[1], wnk.shape[2]
+    _need(x.dtype == wnk.dtype == out.dtype == torch.bfloat16, "x, wnk and out must be bfloat16")
+    _need(head_proj_mfma_supported(x, heads, in_head, K), "operands outside the matrix-core kernel's")
+    _need(x.shape[0] == out.shape[0] and (heads - 1) * in_head + K <= x.shape[1]
+          and (heads - 1) * out_head + N <= out.shape[1], "a head's numbers must lie inside its row")
+    lib.call("arle_head_proj_mfma", x.data_ptr(), x.stride(0), int(in_head), wnk.data_ptr(), out.data_ptr(),
+             out.stride(0), int(out_head), x.shape[0], heads, K, N, _stream())
     return out
 
 

@@ -78,8 +78,14 @@ class LatentAttention(Part):
         self.proj = Linear(torch.cat([wq, wd], dim=0).contiguous(), rt.weight_tiles)
         self.c_norm = tensors["c_norm"]
         # a matrix a head, stored [inner, outer]: q'_h = q_h W_uk,h (W_uk,h is [D, C] as it lies), out_h = lat_h W_uv,h^T
-        self.uk = tensors["uk"].view(self.H, self.D, self.C)
-        self.uv_t = tensors["uv"].view(self.H, self.Dv, self.C).transpose(1, 2).contiguous()
+        # (the matrix-core form of the product reads the other layout, [outer, inner]; only the one that runs is kept)
+        uk, uv = tensors["uk"].view(self.H, self.D, self.C), tensors["uv"].view(self.H, self.Dv, self.C)
+        self.on_matrix_cores = (uk.dtype == torch.bfloat16 and self.D % 8 == 0 and self.C % 8 == 0 and self.R % 8 == 0
+                                and self.q_width % 8 == 0 and (self.C + self.R) % 8 == 0)
+        if self.on_matrix_cores:
+            self.uk_nk, self.uv_nk = uk.transpose(1, 2).contiguous(), uv
+        else:
+            self.uk, self.uv_t = uk, uv.transpose(1, 2).contiguous()
         self.sink = tensors.get("sink")
         self.o = Linear(tensors["o"], rt.weight_tiles)
 
@@ -88,6 +94,16 @@ class LatentAttention(Part):
             return []
         return [("q_dkv", self.proj.out_features, self.proj.in_features, False, None),
                 ("o", self.o.out_features, self.o.in_features, False, "norm")]
+
+    def _per_head(self, x, which, out, *, in_head, out_head):
+        """out[:, head] = x[:, head] . (W_uk,h or W_uv,h^T), a matrix a head."""
+        if self.on_matrix_cores and ops.head_proj_mfma_supported(x, self.H, in_head, self.D if which == "uk" else self.C):
+            ops.head_proj_mfma(x, self.uk_nk if which == "uk" else self.uv_nk, out, heads=self.H, in_head=in_head, out_head=out_head)
+        elif self.on_matrix_cores:      # operands that are not aligned for it after all: the plain kernel, from a turned copy
+            w = (self.uk_nk if which == "uk" else self.uv_nk).transpose(1, 2).contiguous()
+            ops.head_proj(x, w, out, heads=self.H, in_head=in_head, out_head=out_head)
+        else:
+            ops.head_proj(x, self.uk if which == "uk" else self.uv_t, out, heads=self.H, in_head=in_head, out_head=out_head)
 
     def forward(self, x, batch, cache):
         """x [T, H] -> float32 [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
@@ -103,10 +119,10 @@ class LatentAttention(Part):
                         sin=sin, rotary_dims=rot, positions=batch.positions, slot_of_token=batch.slot_of_token,
                         block_table=cache.block_table, k_pages=cache.pages["k"], v_pages=cache.pages["v"],
                         page_size=cache.page_size)
-        ops.head_proj(q, self.uk, q_full, heads=H, in_head=D + R, out_head=C + R)
+        self._per_head(q, "uk", q_full, in_head=D + R, out_head=C + R)
         latent = torch.empty((x.shape[0], H * C), dtype=x.dtype, device=x.device)
         softcap_attention(q_full, latent, cache, batch, num_q_heads=H, num_kv_heads=1, key_dim=C + R, value_dim=C,
                           scale=self.scale, softcap=0.0, r1=None, r2=None, window=self.window, sink=self.sink)
         heads_out = torch.empty((x.shape[0], H * Dv), dtype=x.dtype, device=x.device)
-        ops.head_proj(latent, self.uv_t, heads_out, heads=H, in_head=C, out_head=Dv)
+        self._per_head(latent, "uv", heads_out, in_head=C, out_head=Dv)
         return self.o(heads_out, out_dtype=torch.float32, partials_ok=True)   # into the 32-bit residual unrounded
