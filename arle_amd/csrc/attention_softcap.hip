@@ -525,7 +525,9 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
     }
   };
 
-  if (HEADS || kCapRowsAhead) {
+  // (with keys of more than 128 and values of more than 128 a second set of tile registers no longer fits a wave's
+  // registers: a decoded row behind 1,024 keys of 256 took 144 us with it)
+  if ((HEADS || kCapRowsAhead) && 2 * KC + VC <= 24) {
     // a decoded row's waves are few and each walks a chain of tiles: the next tile's loads fly while this one is worked
     u32x4_t k_even[2][KC], v_even[VC], k_odd[2][KC], v_odd[VC];
     if (tile_first <= tile_last) load_tile(tile_first, k_even, v_even);
@@ -682,6 +684,8 @@ extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* o
     ARLE_CAP(4, 8);
   } else if (size <= 128) {
     ARLE_CAP(8, 8);
+  } else if (Dv <= 192) {
+    ARLE_CAP(8, 12);
   } else {
     ARLE_CAP(8, 16);
   }

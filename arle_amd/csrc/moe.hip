@@ -320,6 +320,142 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
   }
 }
 
+// ---- the same for many rows --------------------------------------------------------------------
+// With a few hundred rows an expert the form above reads every weight fragment from LDS once for sixteen rows, and LDS
+// is what it waits for.  Here a workgroup takes 64 listed rows and 256 weight rows (128 gate and the 128 matching up
+// columns, or 256 columns of down) a k step, both through LDS, and a wave multiplies all 64 rows by 64 weight rows
+// (32 gate and their 32 up columns): sixteen products for four row and four weight fragments.
+constexpr int kBigCols = 256;       // weight rows of a tile
+constexpr int kBigRows = 64;        // listed rows of a tile
+
+template <bool GATE_UP>
+__global__ __launch_bounds__(256) void moe_expert_tiles_kernel(const bf16* __restrict__ x, long long x_stride,
+                                                               const bf16* __restrict__ w, const int* __restrict__ ids,
+                                                               void* __restrict__ out, int tokens, int top, int N, int K) {
+  __shared__ int list_src[kMoeChunk], list_dst[kMoeChunk];
+  __shared__ int wave_count[4];
+  __shared__ __attribute__((aligned(16))) bf16 wt[kBigCols * kMoeLdsRow];
+  __shared__ __attribute__((aligned(16))) bf16 at[kBigRows * kMoeLdsRow];
+  const int e = blockIdx.z;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n = lane % 16, g = lane / 16;
+  {
+    const int t = blockIdx.x * kMoeChunk + threadIdx.x;
+    int slot = -1;
+    if (t < tokens)
+      for (int k = 0; k < top; ++k)
+        if (ids[static_cast<int64_t>(t) * top + k] == e) slot = k;
+    const unsigned long long chose = __ballot(slot >= 0);
+    if (lane == 0) wave_count[wave] = __popcll(chose);
+    __syncthreads();
+    int before = 0;
+    for (int i = 0; i < wave; ++i) before += wave_count[i];
+    if (slot >= 0) {
+      const int rank = before + __popcll(chose & ((1ull << lane) - 1ull));
+      list_src[rank] = GATE_UP ? t : t * top + slot;
+      list_dst[rank] = t * top + slot;
+    }
+    __syncthreads();
+  }
+  const int rows = wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
+  if (rows == 0) return;
+  const int cols = GATE_UP ? kBigCols / 2 : kBigCols;     // output columns of the tile
+  const int n0 = blockIdx.y * cols;
+  const bf16* we = w + static_cast<int64_t>(e) * (GATE_UP ? 2 : 1) * N * K;
+  // the four weight rows of which this thread copies one piece of 8 into LDS (four lanes a row: whole 64-byte lines):
+  // LDS row r belongs to wave r / 64; of a wave's 64 rows the first 32 are gate columns, the last 32 the matching up
+  // columns
+  const int wpiece = (threadIdx.x % 4) * 8;
+  const bf16* wsrc[4];
+  bool w_in[4];
+#pragma unroll
+  for (int h = 0; h < 4; ++h) {
+    const int r = 64 * h + threadIdx.x / 4;
+    int wcol, wrow_global;
+    if (GATE_UP) {
+      const int within = r % 64;
+      wcol = n0 + (r / 64) * 32 + within % 32;
+      wrow_global = within < 32 ? wcol : N + wcol;
+    } else {
+      wcol = n0 + r;
+      wrow_global = wcol;
+    }
+    w_in[h] = wcol < N;
+    wsrc[h] = we + static_cast<int64_t>(w_in[h] ? wrow_global : 0) * K + wpiece;
+  }
+  const int ar = threadIdx.x / 4, apiece = (threadIdx.x % 4) * 8;     // the row piece of x this thread copies
+  const u32x4_t zero = {0, 0, 0, 0};
+  for (int sub = 0; sub * kBigRows < rows; ++sub) {
+    const bf16* arow = x + static_cast<int64_t>(list_src[min(sub * kBigRows + ar, rows - 1)]) * x_stride;
+    f32x4_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const int live = min(4, (rows - sub * kBigRows + 15) / 16);
+    // two k steps are in flight: the loads of step k + 2 are sent while step k is multiplied
+    u32x4_t a_set[2], w_set[2][4];
+    auto fetch = [&](int k0, u32x4_t& a_to, u32x4_t (&w_to)[4]) {
+      a_to = k0 + apiece < K ? *reinterpret_cast<const u32x4_t*>(arow + k0 + apiece) : zero;
+#pragma unroll
+      for (int h = 0; h < 4; ++h)
+        w_to[h] = (w_in[h] && k0 + wpiece < K) ? *reinterpret_cast<const u32x4_t*>(wsrc[h] + k0) : zero;
+    };
+    auto step = [&](int k0, u32x4_t& a_reg, u32x4_t (&w_reg)[4]) {
+      __syncthreads();      // the tiles before have been read by every wave
+      *reinterpret_cast<u32x4_t*>(&at[ar * kMoeLdsRow + apiece]) = a_reg;
+#pragma unroll
+      for (int h = 0; h < 4; ++h)
+        *reinterpret_cast<u32x4_t*>(&wt[(64 * h + threadIdx.x / 4) * kMoeLdsRow + wpiece]) = w_reg[h];
+      __syncthreads();
+      if (k0 + 64 < K) fetch(k0 + 64, a_reg, w_reg);
+      bf16x8_t a_op[4], b_op[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        a_op[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&at[(16 * i + n) * kMoeLdsRow + 8 * g]));
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        b_op[j] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&wt[(64 * wave + 16 * j + n) * kMoeLdsRow + 8 * g]));
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i < live) {       // sixteen rows of the 64 that hold no listed row are not multiplied
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op[i], b_op[j], acc[i][j], 0, 0, 0);
+        }
+    };
+    fetch(0, a_set[0], w_set[0]);
+    if (32 < K) fetch(32, a_set[1], w_set[1]);
+    for (int k0 = 0; k0 < K; k0 += 64) {
+      step(k0, a_set[0], w_set[0]);
+      if (k0 + 32 < K) step(k0 + 32, a_set[1], w_set[1]);
+    }
+    // acc[i][j][c]: listed row 16 i + 4 g + c of the 64, weight row 16 j + n of the wave's 64
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int rr = sub * kBigRows + 16 * i + 4 * g + c;
+        if (rr >= rows) continue;
+        const int64_t dst = static_cast<int64_t>(list_dst[rr]) * N;
+        if (GATE_UP) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const int col = n0 + wave * 32 + 16 * j + n;
+            const float gt = acc[i][j][c];
+            if (col < N) static_cast<bf16*>(out)[dst + col] = from_float<bf16>(gt / (1.0f + expf(-gt)) * acc[i][j + 2][c]);
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int col = n0 + wave * 64 + 16 * j + n;
+            if (col < N) static_cast<float*>(out)[dst + col] = acc[i][j][c];
+          }
+        }
+      }
+    }
+    __syncthreads();        // before the next 64 rows overwrite the tiles
+  }
+}
+
 }  // namespace arle
 
 using namespace arle;
@@ -374,6 +510,15 @@ extern "C" int arle_moe_expert(const void* x, long long x_stride, const void* w,
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == kBF16 && K % 8 == 0 && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+    if (tokens > 64) {      // rows enough that an expert's list fills tiles of 64
+      const int bcols = gate_up ? kBigCols / 2 : kBigCols;
+      const dim3 bgrid((tokens + kMoeChunk - 1) / kMoeChunk, (N + bcols - 1) / bcols, experts);
+      if (gate_up)
+        moe_expert_tiles_kernel<true><<<bgrid, 256, 0, s>>>(static_cast<const bf16*>(x), x_stride, static_cast<const bf16*>(w), ids, out, tokens, top, N, K);
+      else
+        moe_expert_tiles_kernel<false><<<bgrid, 256, 0, s>>>(static_cast<const bf16*>(x), x_stride, static_cast<const bf16*>(w), ids, out, tokens, top, N, K);
+      return launch_status();
+    }
     const int cols = gate_up ? kMoeCols / 2 : kMoeCols;
     const dim3 mgrid((tokens + kMoeChunk - 1) / kMoeChunk, (N + cols - 1) / cols, experts);
     if (gate_up)
