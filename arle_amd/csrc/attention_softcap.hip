@@ -21,7 +21,7 @@
 
 namespace arle {
 
-constexpr int kCapMaxD = 512;
+constexpr int kCapMaxD = 1024;   // the widest head: a latent attention's keys are its latent and its rotated part together
 
 // One wave a (row, head of q, k or v).  T: the element type of q, k, v and the pages; the loads of a head are typed and
 // unconditional (an element past the head's size reads the head's last one and is dropped).
@@ -540,7 +540,7 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
     }
   } else {
     u32x4_t k_now[2][KC], v_now[VC];
-    for (int tile = tile_first; tile <= tile_last; ++tile) {
+    for (int tile = tile_first; tile <= tile_last; tile += tile_step) {
       load_tile(tile, k_now, v_now);
       work_tile(tile, k_now, v_now);
     }

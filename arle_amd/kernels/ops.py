@@ -1628,7 +1628,7 @@ def attn_softcap_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_
     _need(q.shape == (tokens, num_q_heads * key_dim) and out.shape == (tokens, num_q_heads * value_dim)
           and out.dtype == q.dtype, "q [T, nq*Dk] and out [T, nq*Dv] must be of one type")
     _need(num_kv_heads > 0 and num_q_heads % num_kv_heads == 0, "number of q heads must be a multiple of the kv heads")
-    _need(max(key_dim, value_dim) <= MAX_HEAD_DIM and num_q_heads <= _GRID_Y_MAX, "head sizes or counts out of range")
+    _need(max(key_dim, value_dim) <= CAP_SIMT_MAX_DIM and num_q_heads <= _GRID_Y_MAX, "head sizes or counts out of range")
     _check_kv_pages(k_pages, v_pages, num_kv_heads, page_size, key_dim, value_dim, q.dtype)
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
           "block_table must be contiguous int32 [slots, pages]")
@@ -1658,6 +1658,7 @@ def mask_span(window: int, chunk: int) -> int:
 
 
 CAP_MFMA_MAX_DIM = 256
+CAP_SIMT_MAX_DIM = 1024     # the widest head the fixed-order kernel of this family takes
 
 
 def attn_softcap_mfma_supported(dtype, key_dim: int, value_dim: int, page_size: int, group: int) -> bool:

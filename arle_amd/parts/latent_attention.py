@@ -62,9 +62,9 @@ class LatentAttention(Part):
         super().__init__(params, tensors, rt, children)
         self.H, self.D, self.R = int(params["heads"]), int(params["dim"]), int(params["rot_dim"])
         self.Dv, self.C = int(params["value_dim"]), int(params["rank"])
-        if not (0 < self.C + self.R <= ops.MAX_HEAD_DIM):
+        if not (0 < self.C + self.R <= ops.CAP_SIMT_MAX_DIM):
             raise ValueError(f"latent and rotated sizes {self.C} + {self.R} are not supported: the attention kernels "
-                             f"take keys of 1..{ops.MAX_HEAD_DIM}")
+                             f"take keys of 1..{ops.CAP_SIMT_MAX_DIM}")
         if max(self.D, self.C) > ops.HEAD_PROJ_MAX_K:
             raise ValueError(f"head and latent sizes up to {ops.HEAD_PROJ_MAX_K} are taken")
         self.eps = float(params.get("eps", 0.0))
