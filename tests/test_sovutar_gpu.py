@@ -224,7 +224,7 @@ def plain_latent_names(t):
                                     (latent(4, 32, 32, 32, 96, window=37), 16), (latent(20, 16, 16, 16, 48, window=70), 16),
                                     (latent(5, 12, 8, 28, 72, window=19, base=300.0), 16), (latent(2, 8, 4, 8, 16, window=None), 4),
                                     (latent(3, 16, 64, 16, 192, window=45), 16), (latent(18, 8, 16, 8, 144, window=33), 16),
-                                    (latent(2, 16, 64, 16, 512, window=30), 16)])
+                                    (latent(2, 16, 64, 16, 512, window=30, scale=0.05), 16)])
 def test_latent_attention_keeps_its_window_and_its_sink_in_every_cut(dtype, m, page):
     width, T = 56, 100
     window = m["mask"]["size"] if m.get("mask") else None
