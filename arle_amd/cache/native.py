@@ -16,6 +16,7 @@ _ip, _cp = ctypes.POINTER(ctypes.c_int), ctypes.c_char_p
 _SIGNATURES = {
     "arle_group_create": (_p, [_i, _i, _i]),
     "arle_group_destroy": (None, [_p]),
+    "arle_group_set_chunk": (_i, [_p, _i]),
     "arle_group_num_pages": (_i, [_p]),
     "arle_group_free_count": (_i, [_p]),
     "arle_group_held_count": (_i, [_p]),

@@ -96,17 +96,24 @@ class PageGroup:
     The bookkeeping lives in the native runtime core; request keys (any hashable) are mapped to
     integers here."""
 
-    def __init__(self, num_pages: int, page_size: int, window: int | None = None):
+    def __init__(self, num_pages: int, page_size: int, window: int | None = None, chunk: int | None = None):
+        """chunk: queries read only the keys of their own chunk of so many positions (counted from position 0), so the
+        pages in front of the newest chunk go back like those a window has passed."""
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         if window is not None and window <= 0:
             raise ValueError("window must be positive")
+        if chunk is not None and chunk <= 0:
+            raise ValueError("chunk must be positive")
         if num_pages < 0:
             raise ValueError("num_pages must not be negative")
         self.page_size = page_size
         self.window = window
         self._lib = native.lib()
+        self.chunk = chunk
         self._h = self._lib.arle_group_create(num_pages, page_size, window or 0)
+        if chunk is not None:
+            self._lib.arle_group_set_chunk(self._h, int(chunk))
         self.pool = PagePool(num_pages, _handle=self._h)
         self._ids: dict = {}     # request key -> native id
         self._next_id = 0
@@ -171,7 +178,7 @@ class PageGroup:
 
     def trim(self, key) -> list:
         """Give back the pages every key of which the window has passed; returns their logical indices."""
-        if self.window is None:
+        if self.window is None and self.chunk is None:
             return []
         kid = self._id(key)
         cap = len(self._snapshot(key).pages)

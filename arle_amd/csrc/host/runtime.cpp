@@ -67,6 +67,7 @@ struct Table {
 struct Group {
   int page_size;
   int window;  // 0: none
+  int chunk = 0;  // 0: none; else queries read only the keys of their own chunk of so many positions
   Pool pool;
   std::unordered_map<long long, Table> tables;
   Group(int num_pages, int page_size_, int window_) : page_size(page_size_), window(window_), pool(num_pages) {}
@@ -88,6 +89,14 @@ void* arle_group_create(int num_pages, int page_size, int window) {
   return new Group(num_pages, page_size, window);
 }
 void arle_group_destroy(void* h) { delete G(h); }
+
+// Queries of this group read only the keys of their own chunk of `chunk` positions (chunks counted from position 0):
+// `arle_group_trim` then also gives back the pages in front of the chunk that the next query falls into.  0: no chunks.
+int arle_group_set_chunk(void* h, int chunk) {
+  if (chunk < 0) return -1;
+  G(h)->chunk = chunk;
+  return 0;
+}
 
 int arle_group_num_pages(void* h) { return G(h)->pool.num_pages; }
 int arle_group_free_count(void* h) { return static_cast<int>(G(h)->pool.free_.size()); }
@@ -168,15 +177,18 @@ int arle_group_truncate(void* h, long long key, int new_length, int* logical, in
   return dropped;
 }
 
-// Give back the pages every key of which the window has passed.  After `length` tokens the next query sits
+// Give back the pages every key of which the window (or the chunk rule) has passed.  After `length` tokens the next query sits
 // at position >= length and reads keys > position - window, so key c is dead once c <= length - window.
 int arle_group_trim(void* h, long long key, int* logical, int cap) {
   Group* g = G(h);
   auto it = g->tables.find(key);
   if (it == g->tables.end()) return kUnknownKey;
-  if (g->window == 0) return 0;
+  if (g->window == 0 && g->chunk == 0) return 0;
   Table& t = it->second;
-  int dead = std::max(0, t.length - g->window + 1) / g->page_size;
+  int dead = 0;
+  if (g->window > 0) dead = std::max(0, t.length - g->window + 1) / g->page_size;
+  // the next query sits at position `length`, in the chunk that starts at floor(length / chunk) * chunk
+  if (g->chunk > 0) dead = std::max(dead, (t.length / g->chunk * g->chunk) / g->page_size);
   dead = std::min(dead, static_cast<int>(t.pages.size()));
   int n = 0;
   for (int i = t.first_live; i < dead; ++i) {

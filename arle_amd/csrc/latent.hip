@@ -207,7 +207,7 @@ extern "C" int arle_head_proj(const void* in, long long in_stride, int in_head, 
                               long long out_stride, int out_head, int dtype, int rows, int heads, int K, int N,
                               void* stream) {
   if (rows == 0) return 0;
-  if (heads < 1 || heads > 65535 || K < 1 || K > 2048 || N < 1) return static_cast<int>(hipErrorInvalidValue);
+  if (heads < 1 || heads > 65535 || K < 1 || K > 1024 || N < 1) return static_cast<int>(hipErrorInvalidValue);
   const dim3 grid((rows + kProjRows - 1) / kProjRows, heads, (N + kProjThreads - 1) / kProjThreads);
   const size_t lds = static_cast<size_t>(kProjRows) * K * sizeof(float);
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -216,7 +216,7 @@ extern "C" int arle_head_proj(const void* in, long long in_stride, int in_head, 
     static bool raised = false;                                                                                    \
     if (!raised && lds > 48 * 1024) {                                                                              \
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&head_proj_kernel<TT>),               \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kProjRows * 2048 * 4);  \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kProjRows * 1024 * 4);  \
       if (e != hipSuccess) return static_cast<int>(e);                                                             \
       raised = true;                                                                                               \
     }                                                                                                              \

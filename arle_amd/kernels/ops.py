@@ -1818,7 +1818,7 @@ def tanh_cap_(x: torch.Tensor, cap: float) -> torch.Tensor:
 
 # ------------------------------------------------------------------ latent attention's operands
 
-HEAD_PROJ_MAX_K = 2048
+HEAD_PROJ_MAX_K = 1024
 
 
 def latent_prep(q, dkv, q_full, *, heads: int, dim: int, rot_dim: int, rank: int, c_weight, eps: float, cos, sin,

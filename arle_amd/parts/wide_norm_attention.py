@@ -53,7 +53,7 @@ class WideNormAttention(Part):
     @classmethod
     def declare_cache(cls, params):
         nkv, dk, dv = int(params["num_kv_heads"]), int(params["key_dim"]), int(params["value_dim"])
-        return PagedNeed(window=params.get("window"),
+        return PagedNeed(window=params.get("window"), chunk=params.get("chunk"),
                          tensors=(PageTensor("k", (nkv, PAGE, dk)), PageTensor("v", (nkv, dv, PAGE))))
 
     def cache_need(self):

@@ -49,6 +49,28 @@ def test_token_to_page_map_and_truncate():
     g.check()
 
 
+def test_pages_in_front_of_the_newest_chunk_are_given_back():
+    g = PageGroup(num_pages=8, page_size=4, chunk=10)
+    g.open("a")
+    g.append("a", 9)          # keys 0..8; the next query, at 9, is still in chunk 0
+    assert g.trim("a") == []
+    g.append("a", 1)          # length 10: the next query opens chunk 1 and reads keys >= 10; pages 0 and 1 hold keys 0..7
+    assert g.trim("a") == [0, 1]
+    assert g.tables["a"].pages[:2] == [FREED, FREED] and g.pool.free_count == 8 - 1
+    g.append("a", 13)         # length 23: chunk 2 starts at 20: pages 2..4 (keys 8..19) go, page 5 holds keys 20..23
+    assert g.trim("a") == [2, 3, 4]
+    g.check()
+    both = PageGroup(num_pages=8, page_size=4, window=6, chunk=16)
+    both.open("b")
+    both.append("b", 15)      # the window alone: keys <= 15 - 6 are dead, pages 0 and 1
+    assert both.trim("b") == [0, 1]
+    both.append("b", 1)       # length 16: the chunk rule takes every page in front of key 16
+    assert both.trim("b") == [2, 3]
+    both.close("b")
+    g.close("a")
+    assert g.pool.free_count == 8
+
+
 def test_window_pages_are_given_back_while_the_request_runs():
     g = PageGroup(num_pages=6, page_size=4, window=6)
     g.open("a")

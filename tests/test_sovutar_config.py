@@ -49,6 +49,7 @@ def test_the_cache_holds_one_latent_a_token_and_windows_give_pages_back():
     assert all(isinstance(n, PagedNeed) for n in needs)
     lat = raw["layers"][1]["mixer"]
     assert needs[1].window == lat["mask"]["size"] and needs[0].window is None
+    assert needs[0].chunk == raw["layers"][0]["mixer"]["mask"]["size"] and needs[1].chunk is None
     shapes = {t.name: t.page_shape(4) for t in needs[1].page_tensors()}
     assert shapes == {"k": (1, 4, lat["kv_rank"] + lat["rot_dim"]), "v": (1, lat["kv_rank"], 4)}
     per_token = sum(2 * (l["mixer"]["kv_rank"] * 2 + l["mixer"]["rot_dim"]) if l["type"] == "latent_attention"

@@ -432,6 +432,27 @@ def test_bfloat16_rows_do_not_depend_on_the_cut_or_the_batch_beyond_rounding(fol
         assert flipped <= (0 if name in NO_CLOSE_CALLS else 0.05 * total), f"{name} {how}: {flipped} of {total} rows differ"
 
 
+def test_pages_behind_a_chunk_and_a_window_go_back_while_the_request_runs(folders):
+    from arle_amd.cache import FREED
+
+    cfg, weights = read_folder(folders["P"])
+    toks = random_tokens(61, cfg["vocab"], 77)
+    eng = engine_for(folders["P"], "P", "float32", 128)
+    got = replay.run_steps(eng, [{"entries": [("a", toks[:57], list(range(57)))], "end": []}])
+    page = TINY["P"][1]
+    held = {}
+    for group in eng.cache.groups:
+        pages = group.tables["a"].pages
+        held[(group.window, group.chunk)] = sum(p != FREED for p in pages)
+        if group.chunk:      # every page in front of the chunk that position 57 falls into has gone back
+            assert all(p == FREED for p in pages[:(57 // group.chunk * group.chunk) // page])
+    assert held[(None, 11)] == -(-57 // page) - 55 // page and held[(None, 30)] == -(-57 // page) - 30 // page
+    assert held[(9, None)] == -(-57 // page) - (57 - 9 + 1) // page
+    for i in range(57, 61):      # and what follows still equals the plain logits
+        got.update(replay.run_steps(eng, [{"entries": [("a", toks[i:i + 1], [0])], "end": ["a"] if i == 60 else []}]))
+    replay.check_rows(got, {"a": plain.forward(cfg, weights, toks)}, MODEL_TOL["float32"], "after pages went back")
+
+
 def test_captured_steps_give_the_bits_of_eager_ones(folders):
     cfg, _ = read_folder(folders["P"])
     reqs = requests_for(cfg, (30, 30, 41), 300)
