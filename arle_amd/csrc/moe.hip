@@ -321,25 +321,32 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
 }
 
 // ---- the same for many rows --------------------------------------------------------------------
-// With a few hundred rows an expert the form above reads every weight fragment from LDS once for sixteen rows, and LDS
-// is what it waits for.  Here a workgroup takes 64 listed rows and 256 weight rows (128 gate and the 128 matching up
-// columns, or 256 columns of down) a k step, both through LDS, and a wave multiplies all 64 rows by 64 weight rows
-// (32 gate and their 32 up columns): sixteen products for four row and four weight fragments.
+// With a few hundred rows an expert the form above reads every weight fragment from LDS once for sixteen rows, and
+// what a launch waits for is the passes over the weights: every workgroup streams its weight tile over all of K.  Here
+// a workgroup of RG x 4 waves looks through RG x 256 rows of the step and takes RG x 64 listed rows and 256 weight rows
+// (128 gate and the 128 matching up columns, or 256 columns of down) a k step, both through LDS: the weight tile is
+// fetched once for all RG groups of 64 rows, and a wave multiplies the 64 rows of its group by 64 weight rows (32
+// gate and their 32 up columns): sixteen products for four row and four weight fragments.  Two k steps of loads are
+// in flight; sixteen rows that hold no listed row are not multiplied.
 constexpr int kBigCols = 256;       // weight rows of a tile
-constexpr int kBigRows = 64;        // listed rows of a tile
+constexpr int kBigRows = 64;        // listed rows of a group of four waves
 
-template <bool GATE_UP>
-__global__ __launch_bounds__(256) void moe_expert_tiles_kernel(const bf16* __restrict__ x, long long x_stride,
-                                                               const bf16* __restrict__ w, const int* __restrict__ ids,
-                                                               void* __restrict__ out, int tokens, int top, int N, int K) {
-  __shared__ int list_src[kMoeChunk], list_dst[kMoeChunk];
-  __shared__ int wave_count[4];
+template <bool GATE_UP, int RG>
+__global__ __launch_bounds__(256 * RG) void moe_expert_tiles_kernel(const bf16* __restrict__ x, long long x_stride,
+                                                                    const bf16* __restrict__ w, const int* __restrict__ ids,
+                                                                    void* __restrict__ out, int tokens, int top, int N,
+                                                                    int K) {
+  constexpr int kThreads = 256 * RG, kWaves = 4 * RG, kRows = kBigRows * RG;
+  constexpr int kWPieces = kBigCols * 4 / kThreads;      // pieces of 8 of the weight tile a thread copies: 4 / RG
+  __shared__ int list_src[kThreads], list_dst[kThreads];
+  __shared__ int wave_count[kWaves];
   __shared__ __attribute__((aligned(16))) bf16 wt[kBigCols * kMoeLdsRow];
-  __shared__ __attribute__((aligned(16))) bf16 at[kBigRows * kMoeLdsRow];
+  __shared__ __attribute__((aligned(16))) bf16 at[kRows * kMoeLdsRow];
   const int e = blockIdx.z;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n = lane % 16, g = lane / 16;
+  const int rg = wave / 4, cw = wave % 4;     // the wave's group of 64 rows, and its 64 weight rows of the tile
   {
-    const int t = blockIdx.x * kMoeChunk + threadIdx.x;
+    const int t = blockIdx.x * kThreads + threadIdx.x;
     int slot = -1;
     if (t < tokens)
       for (int k = 0; k < top; ++k)
@@ -356,20 +363,22 @@ __global__ __launch_bounds__(256) void moe_expert_tiles_kernel(const bf16* __res
     }
     __syncthreads();
   }
-  const int rows = wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
+  int rows = 0;
+#pragma unroll
+  for (int i = 0; i < kWaves; ++i) rows += wave_count[i];
   if (rows == 0) return;
   const int cols = GATE_UP ? kBigCols / 2 : kBigCols;     // output columns of the tile
   const int n0 = blockIdx.y * cols;
   const bf16* we = w + static_cast<int64_t>(e) * (GATE_UP ? 2 : 1) * N * K;
-  // the four weight rows of which this thread copies one piece of 8 into LDS (four lanes a row: whole 64-byte lines):
-  // LDS row r belongs to wave r / 64; of a wave's 64 rows the first 32 are gate columns, the last 32 the matching up
+  // the weight rows of which this thread copies one piece of 8 into LDS (four lanes a row: whole 64-byte lines):
+  // LDS row r belongs to column wave r / 64; of its 64 rows the first 32 are gate columns, the last 32 the matching up
   // columns
-  const int wpiece = (threadIdx.x % 4) * 8;
-  const bf16* wsrc[4];
-  bool w_in[4];
+  const int piece = (threadIdx.x % 4) * 8;
+  const bf16* wsrc[kWPieces];
+  bool w_in[kWPieces];
 #pragma unroll
-  for (int h = 0; h < 4; ++h) {
-    const int r = 64 * h + threadIdx.x / 4;
+  for (int h = 0; h < kWPieces; ++h) {
+    const int r = (kThreads / 4) * h + static_cast<int>(threadIdx.x) / 4;
     int wcol, wrow_global;
     if (GATE_UP) {
       const int within = r % 64;
@@ -380,41 +389,43 @@ __global__ __launch_bounds__(256) void moe_expert_tiles_kernel(const bf16* __res
       wrow_global = wcol;
     }
     w_in[h] = wcol < N;
-    wsrc[h] = we + static_cast<int64_t>(w_in[h] ? wrow_global : 0) * K + wpiece;
+    wsrc[h] = we + static_cast<int64_t>(w_in[h] ? wrow_global : 0) * K + piece;
   }
-  const int ar = threadIdx.x / 4, apiece = (threadIdx.x % 4) * 8;     // the row piece of x this thread copies
+  const int ar = threadIdx.x / 4;     // the listed row of the tile of which this thread copies one piece
   const u32x4_t zero = {0, 0, 0, 0};
-  for (int sub = 0; sub * kBigRows < rows; ++sub) {
-    const bf16* arow = x + static_cast<int64_t>(list_src[min(sub * kBigRows + ar, rows - 1)]) * x_stride;
+  for (int sub = 0; sub * kRows < rows; ++sub) {
+    const bf16* arow = x + static_cast<int64_t>(list_src[min(sub * kRows + ar, rows - 1)]) * x_stride + piece;
     f32x4_t acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    const int live = min(4, (rows - sub * kBigRows + 15) / 16);
+    const int first = sub * kRows + kBigRows * rg;        // the first listed row of this wave's group
+    const int live = max(0, min(4, (rows - first + 15) / 16));
     // two k steps are in flight: the loads of step k + 2 are sent while step k is multiplied
-    u32x4_t a_set[2], w_set[2][4];
-    auto fetch = [&](int k0, u32x4_t& a_to, u32x4_t (&w_to)[4]) {
-      a_to = k0 + apiece < K ? *reinterpret_cast<const u32x4_t*>(arow + k0 + apiece) : zero;
+    u32x4_t a_set[2], w_set[2][kWPieces];
+    auto fetch = [&](int k0, u32x4_t& a_to, u32x4_t (&w_to)[kWPieces]) {
+      a_to = k0 + piece < K ? *reinterpret_cast<const u32x4_t*>(arow + k0) : zero;
 #pragma unroll
-      for (int h = 0; h < 4; ++h)
-        w_to[h] = (w_in[h] && k0 + wpiece < K) ? *reinterpret_cast<const u32x4_t*>(wsrc[h] + k0) : zero;
+      for (int h = 0; h < kWPieces; ++h)
+        w_to[h] = (w_in[h] && k0 + piece < K) ? *reinterpret_cast<const u32x4_t*>(wsrc[h] + k0) : zero;
     };
-    auto step = [&](int k0, u32x4_t& a_reg, u32x4_t (&w_reg)[4]) {
+    auto step = [&](int k0, u32x4_t& a_reg, u32x4_t (&w_reg)[kWPieces]) {
       __syncthreads();      // the tiles before have been read by every wave
-      *reinterpret_cast<u32x4_t*>(&at[ar * kMoeLdsRow + apiece]) = a_reg;
+      *reinterpret_cast<u32x4_t*>(&at[ar * kMoeLdsRow + piece]) = a_reg;
 #pragma unroll
-      for (int h = 0; h < 4; ++h)
-        *reinterpret_cast<u32x4_t*>(&wt[(64 * h + threadIdx.x / 4) * kMoeLdsRow + wpiece]) = w_reg[h];
+      for (int h = 0; h < kWPieces; ++h)
+        *reinterpret_cast<u32x4_t*>(&wt[((kThreads / 4) * h + static_cast<int>(threadIdx.x) / 4) * kMoeLdsRow + piece]) = w_reg[h];
       __syncthreads();
       if (k0 + 64 < K) fetch(k0 + 64, a_reg, w_reg);
+      if (live == 0) return;
       bf16x8_t a_op[4], b_op[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        a_op[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&at[(16 * i + n) * kMoeLdsRow + 8 * g]));
+        a_op[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&at[(kBigRows * rg + 16 * i + n) * kMoeLdsRow + 8 * g]));
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        b_op[j] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&wt[(64 * wave + 16 * j + n) * kMoeLdsRow + 8 * g]));
+        b_op[j] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&wt[(64 * cw + 16 * j + n) * kMoeLdsRow + 8 * g]));
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         if (i < live) {       // sixteen rows of the 64 that hold no listed row are not multiplied
@@ -428,31 +439,31 @@ __global__ __launch_bounds__(256) void moe_expert_tiles_kernel(const bf16* __res
       step(k0, a_set[0], w_set[0]);
       if (k0 + 32 < K) step(k0 + 32, a_set[1], w_set[1]);
     }
-    // acc[i][j][c]: listed row 16 i + 4 g + c of the 64, weight row 16 j + n of the wave's 64
+    // acc[i][j][c]: listed row 16 i + 4 g + c of the group's 64, weight row 16 j + n of the wave's 64
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const int rr = sub * kBigRows + 16 * i + 4 * g + c;
+        const int rr = first + 16 * i + 4 * g + c;
         if (rr >= rows) continue;
         const int64_t dst = static_cast<int64_t>(list_dst[rr]) * N;
         if (GATE_UP) {
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            const int col = n0 + wave * 32 + 16 * j + n;
+            const int col = n0 + cw * 32 + 16 * j + n;
             const float gt = acc[i][j][c];
             if (col < N) static_cast<bf16*>(out)[dst + col] = from_float<bf16>(gt / (1.0f + expf(-gt)) * acc[i][j + 2][c]);
           }
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const int col = n0 + wave * 64 + 16 * j + n;
+            const int col = n0 + cw * 64 + 16 * j + n;
             if (col < N) static_cast<float*>(out)[dst + col] = acc[i][j][c];
           }
         }
       }
     }
-    __syncthreads();        // before the next 64 rows overwrite the tiles
+    __syncthreads();        // before the next rows overwrite the tiles
   }
 }
 
@@ -512,11 +523,20 @@ extern "C" int arle_moe_expert(const void* x, long long x_stride, const void* w,
       reinterpret_cast<uintptr_t>(w) % 16 == 0) {
     if (tokens > 64) {      // rows enough that an expert's list fills tiles of 64
       const int bcols = gate_up ? kBigCols / 2 : kBigCols;
-      const dim3 bgrid((tokens + kMoeChunk - 1) / kMoeChunk, (N + bcols - 1) / bcols, experts);
-      if (gate_up)
-        moe_expert_tiles_kernel<true><<<bgrid, 256, 0, s>>>(static_cast<const bf16*>(x), x_stride, static_cast<const bf16*>(w), ids, out, tokens, top, N, K);
-      else
-        moe_expert_tiles_kernel<false><<<bgrid, 256, 0, s>>>(static_cast<const bf16*>(x), x_stride, static_cast<const bf16*>(w), ids, out, tokens, top, N, K);
+      const bf16* xb = static_cast<const bf16*>(x);
+      const bf16* wb = static_cast<const bf16*>(w);
+#define ARLE_TILES(GU, RGS)                                                                                      \
+  moe_expert_tiles_kernel<GU, RGS><<<dim3((tokens + 256 * RGS - 1) / (256 * RGS), (N + bcols - 1) / bcols, experts), \
+                                     256 * RGS, 0, s>>>(xb, x_stride, wb, ids, out, tokens, top, N, K)
+      // more rows a weight tile the more rows the step has: a tile's fetch is what the launch waits for
+      if (tokens > 1024) {
+        if (gate_up) ARLE_TILES(true, 4); else ARLE_TILES(false, 4);
+      } else if (tokens > 256) {
+        if (gate_up) ARLE_TILES(true, 2); else ARLE_TILES(false, 2);
+      } else {
+        if (gate_up) ARLE_TILES(true, 1); else ARLE_TILES(false, 1);
+      }
+#undef ARLE_TILES
       return launch_status();
     }
     const int cols = gate_up ? kMoeCols / 2 : kMoeCols;
