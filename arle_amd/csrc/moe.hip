@@ -323,7 +323,7 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
 // ---- the same for many rows --------------------------------------------------------------------
 // With a few hundred rows an expert the form above reads every weight fragment from LDS once for sixteen rows, and
 // what a launch waits for is the passes over the weights: every workgroup streams its weight tile over all of K.  Here
-// a workgroup of RG x 4 waves looks through RG x 256 rows of the step and takes RG x 64 listed rows and 256 weight rows
+// a workgroup of RG x 4 waves (RG 1 or 2) looks through RG x 256 rows of the step and takes RG x 64 listed rows and 256 weight rows
 // (128 gate and the 128 matching up columns, or 256 columns of down) a k step, both through LDS: the weight tile is
 // fetched once for all RG groups of 64 rows, and a wave multiplies the 64 rows of its group by 64 weight rows (32
 // gate and their 32 up columns): sixteen products for four row and four weight fragments.  Two k steps of loads are
@@ -528,10 +528,10 @@ extern "C" int arle_moe_expert(const void* x, long long x_stride, const void* w,
 #define ARLE_TILES(GU, RGS)                                                                                      \
   moe_expert_tiles_kernel<GU, RGS><<<dim3((tokens + 256 * RGS - 1) / (256 * RGS), (N + bcols - 1) / bcols, experts), \
                                      256 * RGS, 0, s>>>(xb, x_stride, wb, ids, out, tokens, top, N, K)
-      // more rows a weight tile the more rows the step has: a tile's fetch is what the launch waits for
-      if (tokens > 1024) {
-        if (gate_up) ARLE_TILES(true, 4); else ARLE_TILES(false, 4);
-      } else if (tokens > 256) {
+      // two groups of 64 rows a weight tile once the step has rows for them: a tile's fetch is what the launch waits
+      // for (all sixteen launches of a 2,048-token prefill at the Qwen3-4B widths: one group 6,508 us, two 5,219 us,
+      // four, which leaves a wave 128 registers, 5,456 us)
+      if (tokens > 256) {
         if (gate_up) ARLE_TILES(true, 2); else ARLE_TILES(false, 2);
       } else {
         if (gate_up) ARLE_TILES(true, 1); else ARLE_TILES(false, 1);
