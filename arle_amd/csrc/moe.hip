@@ -326,22 +326,27 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
 // a workgroup of RG x 4 waves (RG 1 or 2) looks through RG x 256 rows of the step and takes RG x 64 listed rows and 256 weight rows
 // (128 gate and the 128 matching up columns, or 256 columns of down) a k step, both through LDS: the weight tile is
 // fetched once for all RG groups of 64 rows, and a wave multiplies the 64 rows of its group by 64 weight rows (32
-// gate and their 32 up columns): sixteen products for four row and four weight fragments.  Two k steps of loads are
-// in flight; sixteen rows that hold no listed row are not multiplied.
+// gate and their 32 up columns): sixteen products for four row and four weight fragments, twice a k step of 64.  Two
+// k steps of loads are in flight; sixteen rows that hold no listed row are not multiplied.  (A k step of 64 instead
+// of 32, with half the barriers a product: 4,647 instead of 5,228 us for the sixteen launches of a 2,048-token prefill
+// at the Qwen3-4B widths.)
 constexpr int kBigCols = 256;       // weight rows of a tile
 constexpr int kBigRows = 64;        // listed rows of a group of four waves
 
-template <bool GATE_UP, int RG>
+template <bool GATE_UP, int RG, int BK>
 __global__ __launch_bounds__(256 * RG) void moe_expert_tiles_kernel(const bf16* __restrict__ x, long long x_stride,
                                                                     const bf16* __restrict__ w, const int* __restrict__ ids,
                                                                     void* __restrict__ out, int tokens, int top, int N,
                                                                     int K) {
   constexpr int kThreads = 256 * RG, kWaves = 4 * RG, kRows = kBigRows * RG;
-  constexpr int kWPieces = kBigCols * 4 / kThreads;      // pieces of 8 of the weight tile a thread copies: 4 / RG
+  constexpr int kLdsRow = BK + 8;                 // bfloat16 a row of BK takes in LDS (no two lanes of a read on one bank)
+  constexpr int kLanesRow = BK / 8;               // lanes that copy one row of a tile, a piece of 8 each (whole lines)
+  constexpr int kPass = kThreads / kLanesRow;     // rows that the workgroup copies in one go
+  constexpr int kWPieces = kBigCols / kPass, kAPieces = kRows / kPass;
   __shared__ int list_src[kThreads], list_dst[kThreads];
   __shared__ int wave_count[kWaves];
-  __shared__ __attribute__((aligned(16))) bf16 wt[kBigCols * kMoeLdsRow];
-  __shared__ __attribute__((aligned(16))) bf16 at[kRows * kMoeLdsRow];
+  __shared__ __attribute__((aligned(16))) bf16 wt[kBigCols * kLdsRow];
+  __shared__ __attribute__((aligned(16))) bf16 at[kRows * kLdsRow];
   const int e = blockIdx.z;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n = lane % 16, g = lane / 16;
   const int rg = wave / 4, cw = wave % 4;     // the wave's group of 64 rows, and its 64 weight rows of the tile
@@ -370,15 +375,14 @@ __global__ __launch_bounds__(256 * RG) void moe_expert_tiles_kernel(const bf16* 
   const int cols = GATE_UP ? kBigCols / 2 : kBigCols;     // output columns of the tile
   const int n0 = blockIdx.y * cols;
   const bf16* we = w + static_cast<int64_t>(e) * (GATE_UP ? 2 : 1) * N * K;
-  // the weight rows of which this thread copies one piece of 8 into LDS (four lanes a row: whole 64-byte lines):
-  // LDS row r belongs to column wave r / 64; of its 64 rows the first 32 are gate columns, the last 32 the matching up
-  // columns
-  const int piece = (threadIdx.x % 4) * 8;
+  // the weight rows of which this thread copies one piece of 8 into LDS: LDS row r belongs to column wave r / 64; of
+  // its 64 rows the first 32 are gate columns, the last 32 the matching up columns
+  const int piece = (static_cast<int>(threadIdx.x) % kLanesRow) * 8, prow = static_cast<int>(threadIdx.x) / kLanesRow;
   const bf16* wsrc[kWPieces];
   bool w_in[kWPieces];
 #pragma unroll
   for (int h = 0; h < kWPieces; ++h) {
-    const int r = (kThreads / 4) * h + static_cast<int>(threadIdx.x) / 4;
+    const int r = kPass * h + prow;
     int wcol, wrow_global;
     if (GATE_UP) {
       const int within = r % 64;
@@ -391,10 +395,12 @@ __global__ __launch_bounds__(256 * RG) void moe_expert_tiles_kernel(const bf16* 
     w_in[h] = wcol < N;
     wsrc[h] = we + static_cast<int64_t>(w_in[h] ? wrow_global : 0) * K + piece;
   }
-  const int ar = threadIdx.x / 4;     // the listed row of the tile of which this thread copies one piece
   const u32x4_t zero = {0, 0, 0, 0};
   for (int sub = 0; sub * kRows < rows; ++sub) {
-    const bf16* arow = x + static_cast<int64_t>(list_src[min(sub * kRows + ar, rows - 1)]) * x_stride + piece;
+    const bf16* asrc[kAPieces];
+#pragma unroll
+    for (int h = 0; h < kAPieces; ++h)
+      asrc[h] = x + static_cast<int64_t>(list_src[min(sub * kRows + kPass * h + prow, rows - 1)]) * x_stride + piece;
     f32x4_t acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -403,41 +409,46 @@ __global__ __launch_bounds__(256 * RG) void moe_expert_tiles_kernel(const bf16* 
     const int first = sub * kRows + kBigRows * rg;        // the first listed row of this wave's group
     const int live = max(0, min(4, (rows - first + 15) / 16));
     // two k steps are in flight: the loads of step k + 2 are sent while step k is multiplied
-    u32x4_t a_set[2], w_set[2][kWPieces];
-    auto fetch = [&](int k0, u32x4_t& a_to, u32x4_t (&w_to)[kWPieces]) {
-      a_to = k0 + piece < K ? *reinterpret_cast<const u32x4_t*>(arow + k0) : zero;
+    u32x4_t a_set[2][kAPieces], w_set[2][kWPieces];
+    auto fetch = [&](int k0, u32x4_t (&a_to)[kAPieces], u32x4_t (&w_to)[kWPieces]) {
+#pragma unroll
+      for (int h = 0; h < kAPieces; ++h)
+        a_to[h] = k0 + piece < K ? *reinterpret_cast<const u32x4_t*>(asrc[h] + k0) : zero;
 #pragma unroll
       for (int h = 0; h < kWPieces; ++h)
         w_to[h] = (w_in[h] && k0 + piece < K) ? *reinterpret_cast<const u32x4_t*>(wsrc[h] + k0) : zero;
     };
-    auto step = [&](int k0, u32x4_t& a_reg, u32x4_t (&w_reg)[kWPieces]) {
+    auto step = [&](int k0, u32x4_t (&a_reg)[kAPieces], u32x4_t (&w_reg)[kWPieces]) {
       __syncthreads();      // the tiles before have been read by every wave
-      *reinterpret_cast<u32x4_t*>(&at[ar * kMoeLdsRow + piece]) = a_reg;
 #pragma unroll
-      for (int h = 0; h < kWPieces; ++h)
-        *reinterpret_cast<u32x4_t*>(&wt[((kThreads / 4) * h + static_cast<int>(threadIdx.x) / 4) * kMoeLdsRow + piece]) = w_reg[h];
+      for (int h = 0; h < kAPieces; ++h) *reinterpret_cast<u32x4_t*>(&at[(kPass * h + prow) * kLdsRow + piece]) = a_reg[h];
+#pragma unroll
+      for (int h = 0; h < kWPieces; ++h) *reinterpret_cast<u32x4_t*>(&wt[(kPass * h + prow) * kLdsRow + piece]) = w_reg[h];
       __syncthreads();
-      if (k0 + 64 < K) fetch(k0 + 64, a_reg, w_reg);
+      if (k0 + 2 * BK < K) fetch(k0 + 2 * BK, a_reg, w_reg);
       if (live == 0) return;
-      bf16x8_t a_op[4], b_op[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        a_op[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&at[(kBigRows * rg + 16 * i + n) * kMoeLdsRow + 8 * g]));
+      for (int kk = 0; kk < BK; kk += 32) {
+        bf16x8_t a_op[4], b_op[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        b_op[j] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&wt[(64 * cw + 16 * j + n) * kMoeLdsRow + 8 * g]));
+        for (int i = 0; i < 4; ++i)
+          a_op[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&at[(kBigRows * rg + 16 * i + n) * kLdsRow + kk + 8 * g]));
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (i < live) {       // sixteen rows of the 64 that hold no listed row are not multiplied
+        for (int j = 0; j < 4; ++j)
+          b_op[j] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&wt[(64 * cw + 16 * j + n) * kLdsRow + kk + 8 * g]));
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op[i], b_op[j], acc[i][j], 0, 0, 0);
-        }
+        for (int i = 0; i < 4; ++i)
+          if (i < live) {       // sixteen rows of the 64 that hold no listed row are not multiplied
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op[i], b_op[j], acc[i][j], 0, 0, 0);
+          }
+      }
     };
     fetch(0, a_set[0], w_set[0]);
-    if (32 < K) fetch(32, a_set[1], w_set[1]);
-    for (int k0 = 0; k0 < K; k0 += 64) {
+    if (BK < K) fetch(BK, a_set[1], w_set[1]);
+    for (int k0 = 0; k0 < K; k0 += 2 * BK) {
       step(k0, a_set[0], w_set[0]);
-      if (k0 + 32 < K) step(k0 + 32, a_set[1], w_set[1]);
+      if (k0 + BK < K) step(k0 + BK, a_set[1], w_set[1]);
     }
     // acc[i][j][c]: listed row 16 i + 4 g + c of the group's 64, weight row 16 j + n of the wave's 64
 #pragma unroll
@@ -526,8 +537,8 @@ extern "C" int arle_moe_expert(const void* x, long long x_stride, const void* w,
       const bf16* xb = static_cast<const bf16*>(x);
       const bf16* wb = static_cast<const bf16*>(w);
 #define ARLE_TILES(GU, RGS)                                                                                      \
-  moe_expert_tiles_kernel<GU, RGS><<<dim3((tokens + 256 * RGS - 1) / (256 * RGS), (N + bcols - 1) / bcols, experts), \
-                                     256 * RGS, 0, s>>>(xb, x_stride, wb, ids, out, tokens, top, N, K)
+  moe_expert_tiles_kernel<GU, RGS, 64><<<dim3((tokens + 256 * RGS - 1) / (256 * RGS), (N + bcols - 1) / bcols, experts), \
+                                         256 * RGS, 0, s>>>(xb, x_stride, wb, ids, out, tokens, top, N, K)
       // two groups of 64 rows a weight tile once the step has rows for them: a tile's fetch is what the launch waits
       // for (all sixteen launches of a 2,048-token prefill at the Qwen3-4B widths: one group 6,508 us, two 5,219 us,
       // four, which leaves a wave 128 registers, 5,456 us)
