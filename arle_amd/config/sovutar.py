@@ -16,7 +16,7 @@ ARCHITECTURE = "Sovutar"
 
 _TOP = (Key("vocab", int), Key("width", int), Key("norm", dict), Key("layers", list),
         Key("logit_softcap", float, default=0.0))
-_ATTENTION = (Key("heads", int), Key("kv_heads", int), Key("dim", int), Key("vdim", int), Key("scale", float),
+_ATTENTION = (Key("heads", int), Key("kv_heads", int, default=None), Key("dim", int), Key("vdim", int), Key("scale", float),
               Key("mask", dict, default=None), Key("v_mix", bool, default=False))
 _LATENT = (Key("heads", int), Key("dim", int), Key("rot_dim", int), Key("vdim", int), Key("kv_rank", int),
            Key("scale", float), Key("mask", dict, default=None), Key("rot", dict))
@@ -136,7 +136,9 @@ def _read_layer(i: int, raw) -> SovutarLayer:
     kind, m = raw["type"], raw["mixer"]
     if kind == "attention":
         a = _sub(m, _ATTENTION, where + ".mixer")
-        mixer = ChunkedAttentionConfig(a["heads"], a["kv_heads"], a["dim"], a["vdim"], a["scale"],
+        # without `kv_heads` every q head has key and value heads of its own
+        mixer = ChunkedAttentionConfig(a["heads"], a["kv_heads"] if a["kv_heads"] is not None else a["heads"], a["dim"],
+                                       a["vdim"], a["scale"],
                                        _mask_size(a["mask"], where + ".mixer"), a["v_mix"])
         _positive(where, heads=mixer.heads, kv_heads=mixer.kv_heads, dim=mixer.dim, vdim=mixer.vdim)
         if mixer.heads % mixer.kv_heads:

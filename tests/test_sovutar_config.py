@@ -86,3 +86,5 @@ def test_a_model_without_a_cap_or_a_mask_is_taken():
     raw = broken(lambda r: (r.pop("logit_softcap"), r["layers"][0]["mixer"].pop("mask"), r["layers"][1]["mixer"].pop("mask")))
     config = SovutarConfig.from_dict(raw)
     assert config.logit_softcap == 0.0 and config.layers[0].mixer.chunk is None and config.layers[1].mixer.window is None
+    raw = broken(lambda r: [l["mixer"].pop("kv_heads") for l in r["layers"] if l["type"] == "attention"])
+    assert all(l.mixer.kv_heads == l.mixer.heads for l in SovutarConfig.from_dict(raw).layers if l.type == "attention")
